@@ -34,13 +34,109 @@ class PlainOps:
         out.copy_(y.to(out.dtype))
         return out
 
-    def silu_gate(self, gate_up, out):
+    def silu_gate(self, gate_up, out, act=None):
         inner = gate_up.shape[1] // 2
         g, u = gate_up[:, :inner].to(self.work), gate_up[:, inner:].to(self.work)
-        out.copy_((g * torch.sigmoid(g) * u).to(out.dtype))
+        if act is None:
+            out.copy_((g * torch.sigmoid(g) * u).to(out.dtype))
+        else:
+            alpha, limit, shift = act
+            g, u = torch.clamp(g, max=limit), torch.clamp(u, min=-limit, max=limit)
+            out.copy_((g * torch.sigmoid(alpha * g) * (u + shift)).to(out.dtype))
         return out
 
-    def rope_store(self, qkv, bias, positions, cos_sin, slots, k_pages, v_pages, n_q, n_kv, head_dim):
+    # ------------------------------------------------------------ several residual streams
+    def embedding_streams(self, ids, table, positions, rates, out):
+        x = table[ids.long()].to(torch.float32)
+        if rates is not None:
+            angles = positions.to(torch.float32)[:, None] * rates[None, :]
+            x = x.clone()
+            x[:, 0::2] += torch.sin(angles)
+            x[:, 1::2] += torch.cos(angles)
+        out.copy_(x[:, None, :].expand_as(out))
+        return out
+
+    def streams_step(self, streams, write, read, gain, eps, out, rows=None, shift=None):
+        x = streams.to(self.work)
+        if write is not None:
+            y = write.y.to(self.work)
+            if write.scale is not None:
+                y = y * write.scale.to(self.work)
+            x = torch.einsum("tsw,sr->trw", x, write.mix.to(self.work)) + write.out.to(self.work)[None, :, None] * y[:, None, :]
+            if rows is None:
+                streams.copy_(x.to(torch.float32))
+                x = streams.to(self.work)
+        if rows is not None:
+            x = x[rows.long()]
+        u = torch.einsum("tsw,s->tw", x, read.to(self.work))
+        h = u / torch.sqrt((u * u).mean(dim=-1, keepdim=True) + eps) * gain.to(self.work)
+        if shift is not None:
+            mu, state, ctx = shift
+            h32 = h.to(torch.float32)
+            shifted = torch.empty_like(h32)
+            self.token_shift(h32, mu, state, ctx.cu_q, ctx.first_position, ctx.state_slots, ctx.entry_of_token, shifted)
+            h = shifted
+        out.copy_(h.to(out.dtype))
+        return out
+
+    fuses_single_shift = True
+
+    def token_shift(self, h, mu, state, cu_q, first_position, state_slots, entry_of_token, out):
+        out.copy_(h.to(out.dtype))
+        for e in range(cu_q.numel() - 1):
+            lo, hi = int(cu_q[e]), int(cu_q[e + 1])
+            if hi <= lo:
+                continue
+            slot = int(state_slots[e])
+            before = torch.zeros_like(h[0]) if int(first_position[e]) == 0 else state[slot].clone()
+            rows = torch.cat([before[None], h[lo:hi - 1]], dim=0).to(self.work)
+            own = h[lo:hi].to(self.work)
+            out[lo:hi] = (own + (rows - own) * mu.to(self.work)).to(out.dtype)
+            state[slot] = h[hi - 1]
+        return out
+
+    # ------------------------------------------------------------------ matrix memory
+    def mlstm_scan(self, qkvg, gates, state, cu_q, first_position, state_slots, out, heads, d, dv, cap):
+        w = self.work
+        size_c, size_n = heads * d * dv, heads * d
+        for e in range(cu_q.numel() - 1):
+            lo, hi = int(cu_q[e]), int(cu_q[e + 1])
+            if hi <= lo:
+                continue
+            slot = int(state_slots[e])
+            row = state[slot].to(w)
+            if int(first_position[e]) == 0:
+                row = torch.zeros_like(row)
+            c = row[:size_c].reshape(heads, d, dv).clone()
+            n = row[size_c:size_c + size_n].reshape(heads, d).clone()
+            m = row[size_c + size_n:].clone()
+            for t in range(lo, hi):
+                q = qkvg[t, :heads * d].to(w).reshape(heads, d) * d ** -0.5
+                k = qkvg[t, heads * d:2 * heads * d].to(w).reshape(heads, d)
+                v = qkvg[t, 2 * heads * d:2 * heads * d + heads * dv].to(w).reshape(heads, dv)
+                i = cap * torch.tanh(gates[t, :heads].to(w) / cap)
+                f = torch.nn.functional.logsigmoid(cap * torch.tanh(gates[t, heads:2 * heads].to(w) / cap))
+                new_m = torch.maximum(f + m, i)
+                keep, take = torch.exp(f + m - new_m), torch.exp(i - new_m)
+                c = keep[:, None, None] * c + take[:, None, None] * k[:, :, None] * v[:, None, :]
+                n = keep[:, None] * n + take[:, None] * k
+                m = new_m
+                floor = torch.maximum((n * q).sum(-1).abs(), torch.exp(-m)) + 1e-6
+                out[t] = (torch.einsum("hdv,hd->hv", c, q) / floor[:, None]).reshape(-1).to(out.dtype)
+            state[slot] = torch.cat([c.reshape(-1), n.reshape(-1), m]).to(state.dtype)
+        return out
+
+    def head_norm_gate(self, read, weight, gate_rows, gate_offset, eps, heads, dv, out):
+        w = self.work
+        o = read.to(w).reshape(-1, heads, dv)
+        o = o / torch.sqrt((o * o).mean(dim=-1, keepdim=True) + eps)
+        gate = gate_rows[:, gate_offset:gate_offset + heads * dv].to(w)
+        out.copy_((o.reshape(-1, heads * dv) * weight.to(w) * torch.sigmoid(gate)).to(out.dtype))
+        return out
+
+    def rope_store(self, qkv, bias, positions, cos_sin, slots, k_pages, v_pages, n_q, n_kv, head_dim, value_dim=None):
+        if value_dim is not None and value_dim != head_dim:
+            return self._store_uneven(qkv, bias, positions, cos_sin, slots, k_pages, v_pages, n_q, n_kv, head_dim, value_dim)
         n_tokens = qkv.shape[0]
         x = qkv.to(self.work)
         if bias is not None:
@@ -65,8 +161,36 @@ class PlainOps:
                 k_pages[page, :, off, :] = stored[t, n_q:n_q + n_kv]
                 v_pages[page, :, :, off] = stored[t, n_q + n_kv:]       # values lie transposed in a page
 
+    def _store_uneven(self, qkv, bias, positions, cos_sin, slots, k_pages, v_pages, n_q, n_kv, d, dv):
+        """Value heads of another size than the key heads: rows are [n_q d | n_kv d | n_kv dv]."""
+        n_tokens = qkv.shape[0]
+        x = qkv.to(self.work)
+        if bias is not None:
+            x = x + bias.to(self.work)
+        rot = x[:, :(n_q + n_kv) * d].reshape(n_tokens, n_q + n_kv, d).clone()
+        if cos_sin is not None:
+            half = d // 2
+            cs = cos_sin[positions.long()].to(self.work)
+            cos, sin = cs[:, None, :half], cs[:, None, half:]
+            x1, x2 = rot[..., :half], rot[..., half:]
+            rot = torch.cat([x1 * cos - x2 * sin, x2 * cos + x1 * sin], dim=-1)
+        x = torch.cat([rot.reshape(n_tokens, -1), x[:, (n_q + n_kv) * d:]], dim=1)
+        qkv.copy_(x.to(qkv.dtype))
+        if slots is not None:
+            page_size = k_pages.shape[2]
+            keys = qkv[:, n_q * d:(n_q + n_kv) * d].reshape(n_tokens, n_kv, d)
+            values = qkv[:, (n_q + n_kv) * d:].reshape(n_tokens, n_kv, dv)
+            for t in range(n_tokens):
+                slot = int(slots[t])
+                if slot < 0:
+                    continue
+                page, off = divmod(slot, page_size)
+                k_pages[page, :, off, :] = keys[t]
+                v_pages[page, :, :, off] = values[t]
+
     def paged_attention(self, qkv, out, k_pages, v_pages, positions, entry_of_token, block_table,
-                        n_q, n_kv, head_dim, window, scale, max_position=None, batch=None):
+                        n_q, n_kv, head_dim, window, scale, max_position=None, batch=None,
+                        value_dim=None, chunk=None, slopes=None, sinks=None):
         page_size = k_pages.shape[2]
         group = n_q // n_kv
         for t in range(qkv.shape[0]):
@@ -75,6 +199,8 @@ class PlainOps:
             pos = int(positions[t])
             table = block_table[int(entry_of_token[t])]
             lo = max(0, pos - window) if window is not None else 0
+            if chunk is not None:
+                lo = max(lo, pos // chunk * chunk)
             keys = list(range(lo, pos + 1))
             pages = [int(table[j // page_size]) for j in keys]
             assert all(p >= 0 for p in pages), "attention reads a page that was given back"
@@ -85,7 +211,15 @@ class PlainOps:
             k = k.repeat_interleave(group, dim=1)            # [keys, n_q, d]
             v = v.repeat_interleave(group, dim=1)
             scores = torch.einsum("hd,khd->hk", q, k) * scale
-            probs = torch.softmax(scores, dim=-1)
+            if slopes is not None:
+                distance = pos - torch.tensor(keys, dtype=self.work)
+                scores = scores - slopes.to(self.work)[:, None] * distance[None, :]
+            if sinks is None:
+                probs = torch.softmax(scores, dim=-1)
+            else:
+                top = torch.maximum(scores.max(dim=-1).values, sinks.to(self.work))
+                e = torch.exp(scores - top[:, None])
+                probs = e / (e.sum(dim=-1) + torch.exp(sinks.to(self.work) - top))[:, None]
             out[t] = torch.einsum("hk,khd->hd", probs, v).reshape(-1).to(out.dtype)
         return out
 
@@ -101,10 +235,10 @@ class PlainOps:
             return out
         return y
 
-    def linear_silu_gate(self, x, weight, out=None):
+    def linear_silu_gate(self, x, weight, out=None, act=None):
         inner = weight.shape[0] // 2
         result = torch.empty((x.shape[0], inner), dtype=x.dtype, device=x.device) if out is None else out
-        return self.silu_gate(self.linear(x, weight), result)
+        return self.silu_gate(self.linear(x, weight), result, act=act)
 
     # The fused decode products, as compositions of the ops above.
     fuse_rows = 16

@@ -148,7 +148,8 @@ class CacheManager:
         self._lib = _host.lib()
         kept = [retention_window(need) for need, _ in planned]
         windows = (ctypes.c_int32 * max(1, len(planned)))(*[-1 if w is None else w for w in kept])
-        self.state_layers = [i for i, need in enumerate(needs) if need.state_shape is not None]
+        self.state_layers = [i for i, need in enumerate(needs)
+                             if need.state_shape is not None or need.block_state_shape is not None]
         self._core = self._lib.ta_cache_new(len(planned), windows, num_pages, page_size, max_requests,
                                             1 if prefix_cache else 0, len(self.state_layers))
         if not self._core:

@@ -2,7 +2,8 @@ from .base import ConfigError, ModelConfig, read_config_json
 from .registry import (Architecture, architecture_name, get_architecture, load_config,
                        register_architecture, registered_architectures)
 from .qwen2 import Qwen2Config
+from .napadra import NapadraConfig
 
 __all__ = ["ConfigError", "ModelConfig", "read_config_json", "Architecture", "architecture_name",
            "get_architecture", "load_config", "register_architecture", "registered_architectures",
-           "Qwen2Config"]
+           "Qwen2Config", "NapadraConfig"]

@@ -1,6 +1,6 @@
 """One registry from an architecture's name to its configuration and model.
 
-The name is `config.json:architectures[0]`.  An architecture registers a
+The name is `config.json:architectures[0]` (or the string `architecture`).  An architecture registers a
 configuration class and a function that turns a configuration into a
 `ModelSpec` (the list of layers, their parts and the order they run in).
 """
@@ -46,10 +46,12 @@ def get_architecture(name: str) -> Architecture:
 
 def architecture_name(raw: dict[str, Any]) -> str:
     names = raw.get("architectures")
-    if not isinstance(names, list) or not names or not isinstance(names[0], str):
-        raise ConfigError("config.json has no `architectures` list naming the model class; registered: "
-                          + ", ".join(registered_architectures()))
-    return names[0]
+    if isinstance(names, list) and names and isinstance(names[0], str):
+        return names[0]
+    if isinstance(raw.get("architecture"), str):       # files that name the one class under `architecture`
+        return raw["architecture"]
+    raise ConfigError("config.json has neither an `architectures` list nor an `architecture` string naming the "
+                      "model class; registered: " + ", ".join(registered_architectures()))
 
 
 def load_config(folder_or_file: str) -> ModelConfig:

@@ -258,6 +258,7 @@ class Engine:
             k_pages, v_pages = self.pools.layer_pages(source)
             self.layer_caches.append(LayerCache(group=self.cache.group_of_layer[source], k_pages=k_pages,
                                                 v_pages=v_pages, state=self.pools.states.get(source),
+                                                block_state=self.pools.block_states.get(entry.layer),
                                                 writes=entry.cache_of is None))
         self.steps = 0
         self._landing: dict[int, tuple] = {}     # pinned rows and events of `decode_greedy` / `decode_sampled`, by batch size

@@ -1,1 +1,2 @@
 from . import qwen2  # noqa: F401  (registers Qwen2ForCausalLM)
+from . import napadra  # noqa: F401  (registers Napadra)

@@ -20,6 +20,13 @@ class GQAttention(Mixer):
     (model.rs:571-580); scores are scaled by 1/sqrt(d) after the product; a key is visible when
     key <= query and, with a window w, key + w >= query (model.rs:119-129).
     The three projection matrices are joined into one at load time so one product makes q, k and v.
+
+    Options of the spec, each on its own: `value_dim` (value heads of another size than the key heads), `chunk`
+    (a query sees only the keys of its own run of `chunk` positions, runs counted from position 0 of the
+    sequence), `distance_bias` b (head h's score loses 2^(-b (h+1) / n_heads) for every position between query
+    and key), `sink` (tensor `sink`, one number per head, joins the softmax's denominator as exp(sink): no key,
+    no value, not scaled, no bias) and `own_kv` False (no key and value projections: the layer reads the pages
+    of the layer it is pointed at and writes nothing).  Scores, bias and weights are float32 in every kernel.
     """
     graph_safe = True
 
@@ -27,12 +34,24 @@ class GQAttention(Mixer):
     def __init__(self, spec: MixerSpec, tensors: dict[str, torch.Tensor], runtime: Runtime):
         self.spec, self.runtime = spec, runtime
         self.n_q, self.n_kv, self.d = spec.n_heads, spec.n_kv_heads, spec.head_dim
-        self.w_qkv = torch.cat([tensors["q_proj.weight"], tensors["k_proj.weight"],
-                                tensors["v_proj.weight"]], dim=0).contiguous()
+        self.dv = spec.value_dim or spec.head_dim
+        self.own_kv = spec.own_kv
+        joined = ("q_proj", "k_proj", "v_proj") if spec.own_kv else ("q_proj",)
+        self.w_qkv = torch.cat([tensors[f"{name}.weight"] for name in joined], dim=0).contiguous()
         self.b_qkv = None
         if spec.qkv_bias:
-            self.b_qkv = torch.cat([tensors["q_proj.bias"], tensors["k_proj.bias"],
-                                    tensors["v_proj.bias"]], dim=0).contiguous()
+            self.b_qkv = torch.cat([tensors[f"{name}.bias"] for name in joined], dim=0).contiguous()
+        self.chunk = spec.chunk
+        self.slopes = None
+        if spec.distance_bias is not None:
+            self.slopes = torch.tensor([2.0 ** (-float(spec.distance_bias) * (h + 1) / self.n_q) for h in range(self.n_q)],
+                                       dtype=torch.float32, device=runtime.device)
+        self.sinks = tensors["sink"].to(torch.float32).contiguous() if spec.sink else None
+        # What the kernels written for the plain form (equal head sizes, every earlier key visible up to a window,
+        # a softmax over the keys alone) do not compute.
+        self.extras = dict(value_dim=self.dv, chunk=self.chunk, slopes=self.slopes, sinks=self.sinks)
+        self.plain = (self.dv == self.d and self.chunk is None and self.slopes is None and self.sinks is None
+                      and self.own_kv)
         self.w_o = tensors["o_proj.weight"]
         self.b_o = tensors.get("o_proj.bias") if spec.out_bias else None
         self.scale = float(spec.scale) if spec.scale is not None else 1.0 / math.sqrt(self.d)
@@ -44,24 +63,33 @@ class GQAttention(Mixer):
     @staticmethod
     def tensor_specs(spec: MixerSpec) -> dict[str, TensorSpec]:
         q_out, kv_out, hidden = spec.n_heads * spec.head_dim, spec.n_kv_heads * spec.head_dim, spec.hidden_size
-        out = {"q_proj.weight": TensorSpec((q_out, hidden)), "k_proj.weight": TensorSpec((kv_out, hidden)),
-               "v_proj.weight": TensorSpec((kv_out, hidden)), "o_proj.weight": TensorSpec((hidden, q_out))}
+        dv = spec.value_dim or spec.head_dim
+        out = {"q_proj.weight": TensorSpec((q_out, hidden)), "o_proj.weight": TensorSpec((hidden, spec.n_heads * dv))}
+        if spec.own_kv:
+            out.update({"k_proj.weight": TensorSpec((kv_out, hidden)),
+                        "v_proj.weight": TensorSpec((spec.n_kv_heads * dv, hidden))})
         if spec.qkv_bias:
-            out.update({"q_proj.bias": TensorSpec((q_out,), role="vector"),
-                        "k_proj.bias": TensorSpec((kv_out,), role="vector"),
-                        "v_proj.bias": TensorSpec((kv_out,), role="vector")})
+            out["q_proj.bias"] = TensorSpec((q_out,), role="vector")
+            if spec.own_kv:
+                out.update({"k_proj.bias": TensorSpec((kv_out,), role="vector"),
+                            "v_proj.bias": TensorSpec((spec.n_kv_heads * dv,), role="vector")})
+        if spec.sink:
+            out["sink"] = TensorSpec((spec.n_heads,), role="vector", std=1.0)
         if spec.out_bias:
             out["o_proj.bias"] = TensorSpec((hidden,), role="vector")
         return out
 
     @staticmethod
     def cache_need(spec: MixerSpec) -> CacheNeed:
+        if not spec.own_kv:
+            return CacheNeed()                  # it reads the pages of the layer it is pointed at
         kind = "full" if spec.window is None else "window"
-        return CacheNeed(kind=kind, n_kv_heads=spec.n_kv_heads, head_dim=spec.head_dim, window=spec.window)
+        return CacheNeed(kind=kind, n_kv_heads=spec.n_kv_heads, head_dim=spec.head_dim, window=spec.window,
+                         value_dim=spec.value_dim or 0)
 
     def repeatable(self):
         position = repeatable_of(self.position)
-        if position is None:
+        if position is None or not self.plain:
             return None
         return Repeatable(("gqa_attention", self.n_q, self.n_kv, self.d, self.scale, self.window, position.constants),
                           (self.w_qkv, self.b_qkv, self.w_o, self.b_o) + position.tensors)
@@ -73,7 +101,7 @@ class GQAttention(Mixer):
         # The norm and the position encoding say themselves whether they have the form the fused kernels compute.
         fold = norm.fold() if delta is None else None
         behind = self.position.epilogue() if fold is not None else None
-        fused = (behind is not None and self.d % 32 == 0 and cache.group is not None
+        fused = (behind is not None and self.d % 32 == 0 and cache.group is not None and self.plain
                  and _can_fuse(ops, residual, self.runtime.dtype))
         if not fused:
             # The output is handed on as a delta: an output product whose K is cut over workgroups may stay in
@@ -100,7 +128,8 @@ class GQAttention(Mixer):
         ops = self.runtime.ops
         can = getattr(ops, "can_rope_store", None)
         behind = None
-        if can and can(x.shape[0], self.runtime.dtype, self.w_qkv.numel()) and self.d % 32 == 0 and cache.group is not None:
+        if (can and can(x.shape[0], self.runtime.dtype, self.w_qkv.numel()) and self.d % 32 == 0
+                and cache.group is not None and self.plain):
             behind = self.position.epilogue()
         if behind is not None:
             # A few dozen rows: bias, rotation and the cache write ride in the projection's epilogue.
@@ -109,9 +138,19 @@ class GQAttention(Mixer):
                                           cache.v_pages, self.n_q, self.n_kv, self.d)
         else:
             qkv = ops.linear(x, self.w_qkv, self.b_qkv)   # bias joins the float accumulator
-            self.position.encode_and_store(qkv, None, self.n_q, self.n_kv, self.d, ctx, cache)
-        mixed = torch.empty((x.shape[0], self.n_q * self.d), dtype=x.dtype, device=x.device)
-        ops.paged_attention(qkv, mixed, cache.k_pages, cache.v_pages, ctx.positions, ctx.entry_of_token,
-                            ctx.block_tables[cache.group], self.n_q, self.n_kv, self.d, self.window,
-                            self.scale, max_position=ctx.max_position, batch=ctx)
+            if self.plain:
+                self.position.encode_and_store(qkv, None, self.n_q, self.n_kv, self.d, ctx, cache)
+            elif self.own_kv:
+                self.position.encode_and_store(qkv, None, self.n_q, self.n_kv, self.d, ctx, cache, value_dim=self.dv)
+            else:                               # queries alone: encoded in place, nothing to store
+                self.position.encode_and_store(qkv, None, self.n_q, 0, self.d, ctx, cache, value_dim=self.dv)
+        mixed = torch.empty((x.shape[0], self.n_q * self.dv), dtype=x.dtype, device=x.device)
+        if self.plain:
+            ops.paged_attention(qkv, mixed, cache.k_pages, cache.v_pages, ctx.positions, ctx.entry_of_token,
+                                ctx.block_tables[cache.group], self.n_q, self.n_kv, self.d, self.window,
+                                self.scale, max_position=ctx.max_position, batch=ctx)
+        else:
+            ops.paged_attention(qkv, mixed, cache.k_pages, cache.v_pages, ctx.positions, ctx.entry_of_token,
+                                ctx.block_tables[cache.group], self.n_q, self.n_kv, self.d, self.window,
+                                self.scale, max_position=ctx.max_position, batch=ctx, **self.extras)
         return ops.linear(mixed, self.w_o, self.b_o, pending=True) if pending else ops.linear(mixed, self.w_o, self.b_o)

@@ -19,9 +19,15 @@ class GatedDense(FeedForward):
 
 
     def __init__(self, spec: FeedForwardSpec, tensors: dict[str, torch.Tensor], runtime: Runtime):
-        if spec.activation != "silu":
-            raise ValueError(f"gated_dense knows the silu activation, not {spec.activation!r}")
+        if spec.activation not in ("silu", "capped_swish"):
+            raise ValueError(f"gated_dense knows the activations silu and capped_swish, not {spec.activation!r}")
         self.spec, self.runtime = spec, runtime
+        # capped_swish: g' = min(g, limit), u' = clamp(u, -limit, limit); g' * sigmoid(alpha g') * (u' + shift).
+        # (silu is alpha 1, no limit, shift 0, and keeps the kernels written for it.)
+        self.act = None
+        if spec.activation == "capped_swish":
+            limit = float("inf") if spec.act_limit is None else float(spec.act_limit)
+            self.act = (float(spec.act_alpha), limit, float(spec.act_up_shift))
         gate, up, down = tensors["gate_proj.weight"], tensors["up_proj.weight"], tensors["down_proj.weight"]
         # The bfloat16 products read eight elements of K at a time.  An inner width that is no multiple of
         # eight is filled up with zero rows of gate and up and zero columns of down: act(0) * 0 = 0 meets a
@@ -41,14 +47,14 @@ class GatedDense(FeedForward):
                 "down_proj.weight": TensorSpec((spec.hidden_size, spec.intermediate_size))}
 
     def repeatable(self):
-        return Repeatable(("gated_dense",), (self.w_gate_up, self.w_down))
+        return Repeatable(("gated_dense", self.act), (self.w_gate_up, self.w_down))
 
     def forward_normed(self, residual, delta, norm, ctx):
         """Decode batches of few bfloat16 rows: norm + gate/up product + activation in one kernel, then the
         down product added straight into the residual stream."""
         ops = self.runtime.ops
         fold = norm.fold() if delta is None else None      # the norm says whether it has the form the kernel computes
-        if fold is None or not _can_fuse(ops, residual, self.runtime.dtype):
+        if fold is None or self.act is not None or not _can_fuse(ops, residual, self.runtime.dtype):
             # The output is handed on as a delta: a down product whose K is cut over workgroups may stay in
             # parts, and the norm that takes it next adds them in its own kernel.
             return self._run(norm.apply(residual, delta), pending=getattr(ops, "takes_pending", False))
@@ -64,5 +70,5 @@ class GatedDense(FeedForward):
 
     def _run(self, x, pending: bool):
         ops = self.runtime.ops
-        act = ops.linear_silu_gate(x, self.w_gate_up)
+        act = ops.linear_silu_gate(x, self.w_gate_up) if self.act is None else ops.linear_silu_gate(x, self.w_gate_up, act=self.act)
         return ops.linear(act, self.w_down, pending=True) if pending else ops.linear(act, self.w_down)

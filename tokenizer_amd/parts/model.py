@@ -10,7 +10,19 @@ from .spec import CacheNeed, ModelSpec, TensorSpec
 
 
 def _prefixed(prefix: str, specs: dict[str, TensorSpec]) -> dict[str, TensorSpec]:
-    return {f"{prefix}.{name}" if prefix else name: spec for name, spec in specs.items()}
+    """(A part's tensor with the empty name is the tensor that the prefix itself names.)"""
+    return {(f"{prefix}.{name}" if name else prefix) if prefix else name: spec for name, spec in specs.items()}
+
+
+def _renamed(specs: dict[str, TensorSpec], names) -> dict[str, TensorSpec]:
+    """A part's tensors under the names a file gives them (`names`: pairs of the part's name and the file's)."""
+    table = dict(names or ())
+    return {table.get(name, name): spec for name, spec in specs.items()}
+
+
+def _named_back(tensors: dict[str, torch.Tensor], names) -> dict[str, torch.Tensor]:
+    table = {theirs: ours for ours, theirs in (names or ())}
+    return {table.get(name, name): value for name, value in tensors.items()}
 
 
 def expected_tensors(spec: ModelSpec) -> dict[str, TensorSpec]:
@@ -30,7 +42,10 @@ def build_model(spec: ModelSpec, tensors: dict[str, torch.Tensor], runtime: Runt
 
 def _strip(prefix: str, tensors: dict[str, torch.Tensor]) -> dict[str, torch.Tensor]:
     lead = prefix + "."
-    return {name[len(lead):]: value for name, value in tensors.items() if name.startswith(lead)}
+    out = {name[len(lead):]: value for name, value in tensors.items() if name.startswith(lead)}
+    if prefix in tensors:
+        out[""] = tensors[prefix]
+    return out
 
 
 @dataclasses.dataclass
@@ -40,6 +55,7 @@ class LayerCache:
     k_pages: torch.Tensor | None = None     # [n_pages, n_kv, page_size, d]
     v_pages: torch.Tensor | None = None
     state: torch.Tensor | None = None       # [n_slots, *state_shape]
+    block_state: torch.Tensor | None = None  # float32 [n_slots, *block_state_shape]: what the block itself keeps
     writes: bool = True                     # False when the layer reads another layer's cache
     makes: dict = dataclasses.field(default_factory=dict, repr=False, compare=False)   # what the layers run on it depend on
 
@@ -127,12 +143,17 @@ class DecoderModel:
         for layer in spec.layers:
             if layer.mixer is not None:
                 out.update(_prefixed(layer.mixer_norm_prefix, NORMS.get(layer.mixer_norm.kind).tensor_specs(layer.mixer_norm)))
-                out.update(_prefixed(layer.mixer_prefix, MIXERS.get(layer.mixer.kind).tensor_specs(layer.mixer)))
+                out.update(_prefixed(layer.mixer_prefix, _renamed(MIXERS.get(layer.mixer.kind).tensor_specs(layer.mixer),
+                                                                  layer.mixer.tensor_names)))
             if layer.feed_forward is not None:
                 out.update(_prefixed(layer.feed_forward_norm_prefix,
                                      NORMS.get(layer.feed_forward_norm.kind).tensor_specs(layer.feed_forward_norm)))
                 out.update(_prefixed(layer.feed_forward_prefix,
-                                     FEED_FORWARDS.get(layer.feed_forward.kind).tensor_specs(layer.feed_forward)))
+                                     _renamed(FEED_FORWARDS.get(layer.feed_forward.kind).tensor_specs(layer.feed_forward),
+                                              layer.feed_forward.tensor_names)))
+            own = getattr(BLOCKS.get(layer.block), "tensor_specs", None)
+            if own is not None:                    # a block with tensors of its own
+                out.update(_prefixed(layer.prefix, own(layer)))
         out.update(_prefixed(spec.final_norm_prefix, NORMS.get(spec.final_norm.kind).tensor_specs(spec.final_norm)))
         if not spec.tied_head:
             out[spec.head_name] = TensorSpec((spec.vocab_size, spec.hidden_size))
@@ -140,9 +161,14 @@ class DecoderModel:
 
     @staticmethod
     def cache_needs(spec: ModelSpec) -> list[CacheNeed]:
-        """(A layer without a mixer asks for nothing.)"""
-        return [MIXERS.get(layer.mixer.kind).cache_need(layer.mixer) if layer.mixer is not None else CacheNeed()
-                for layer in spec.layers]
+        """(A layer without a mixer asks for nothing.  A block that keeps state of its own adds it to the mixer's
+        need: `cache_need(layer, need)`.)"""
+        needs = []
+        for layer in spec.layers:
+            need = MIXERS.get(layer.mixer.kind).cache_need(layer.mixer) if layer.mixer is not None else CacheNeed()
+            own = getattr(BLOCKS.get(layer.block), "cache_need", None)
+            needs.append(need if own is None else own(layer, need))
+        return needs
 
     def __init__(self, spec: ModelSpec, tensors: dict[str, torch.Tensor], runtime: Runtime):
         self.spec, self.runtime = spec, runtime
@@ -152,13 +178,20 @@ class DecoderModel:
             mixer_norm = mixer = ff_norm = feed_forward = None
             if layer.mixer is not None:
                 mixer_norm = NORMS.get(layer.mixer_norm.kind)(layer.mixer_norm, _strip(layer.mixer_norm_prefix, tensors), runtime)
-                mixer = MIXERS.get(layer.mixer.kind)(layer.mixer, _strip(layer.mixer_prefix, tensors), runtime)
+                mixer = MIXERS.get(layer.mixer.kind)(layer.mixer, _named_back(_strip(layer.mixer_prefix, tensors),
+                                                                               layer.mixer.tensor_names), runtime)
             if layer.feed_forward is not None:
                 ff_norm = NORMS.get(layer.feed_forward_norm.kind)(layer.feed_forward_norm,
                                                                   _strip(layer.feed_forward_norm_prefix, tensors), runtime)
-                feed_forward = FEED_FORWARDS.get(layer.feed_forward.kind)(layer.feed_forward,
-                                                                         _strip(layer.feed_forward_prefix, tensors), runtime)
-            self.blocks.append(BLOCKS.get(layer.block)(mixer_norm, mixer, ff_norm, feed_forward))
+                feed_forward = FEED_FORWARDS.get(layer.feed_forward.kind)(
+                    layer.feed_forward, _named_back(_strip(layer.feed_forward_prefix, tensors),
+                                                    layer.feed_forward.tensor_names), runtime)
+            block = BLOCKS.get(layer.block)
+            if hasattr(block, "tensor_specs"):     # a block with tensors and constants of its own is handed them
+                self.blocks.append(block(mixer_norm, mixer, ff_norm, feed_forward, layer=layer,
+                                         tensors=_strip(layer.prefix, tensors), runtime=runtime))
+            else:
+                self.blocks.append(block(mixer_norm, mixer, ff_norm, feed_forward))
         self.final_norm = NORMS.get(spec.final_norm.kind)(spec.final_norm, _strip(spec.final_norm_prefix, tensors), runtime)
         self.head = self.embedding if spec.tied_head else tensors[spec.head_name]
         parts = [self.final_norm] + [p for b in self.blocks if hasattr(b, "mixer")

@@ -33,3 +33,23 @@ class RMSNorm(Norm):
         out = torch.empty((n_rows, self.size), dtype=self.runtime.dtype, device=residual.device)
         return self.runtime.ops.add_rmsnorm(residual, delta, self.weight, self.eps, out, rows,
                                             store_residual=rows is None)
+
+
+@NORMS.register("rmsnorm_scalar")
+class ScalarRMSNorm(RMSNorm):
+    """y = x / sqrt(mean(x^2) + eps) * g with one number g for every coordinate: the tensor that the norm's prefix
+    itself names, of shape [].  `gain` is that number (float32 [1]) for kernels that take it so; `weight` repeats
+    it over the row for the kernels of the norm above, which this norm then shares (its `fold()` too)."""
+    graph_safe = True
+
+    def __init__(self, spec: NormSpec, tensors: dict[str, torch.Tensor], runtime: Runtime):
+        self.size, self.eps, self.runtime = spec.size, float(spec.eps), runtime
+        self.gain = tensors[""].reshape(1).to(torch.float32).contiguous()
+        self.weight = self.gain.expand(spec.size).contiguous()
+
+    @staticmethod
+    def tensor_specs(spec: NormSpec) -> dict[str, TensorSpec]:
+        return {"": TensorSpec((), init="ones", role="vector")}
+
+    def repeatable(self):
+        return Repeatable(("rmsnorm_scalar", self.size, self.eps), (self.weight, self.gain))

@@ -29,11 +29,16 @@ class NoPosition(PositionEncoding):
             return None
         return StoreEpilogue(self.table())
 
-    def encode_and_store(self, qkv, bias, n_q, n_kv, head_dim, ctx, cache):
-        slots = ctx.slots[cache.group] if cache.writes else None
+    def encode_and_store(self, qkv, bias, n_q, n_kv, head_dim, ctx, cache, value_dim=None):
+        """`value_dim`: the size of a value head where it is not `head_dim`.  `n_kv` 0: the rows hold query heads
+        alone and nothing is stored."""
+        slots = ctx.slots[cache.group] if cache.writes and n_kv else None
+        extra = {} if value_dim is None or value_dim == head_dim else {"value_dim": value_dim}
+        if n_kv == 0 and self.table() is None and bias is None:
+            return                              # nothing to add, rotate or store
         self.runtime.ops.rope_store(qkv, bias, ctx.positions, self.table(), slots,
-                                    cache.k_pages if cache.writes else None,
-                                    cache.v_pages if cache.writes else None, n_q, n_kv, head_dim)
+                                    cache.k_pages if slots is not None else None,
+                                    cache.v_pages if slots is not None else None, n_q, n_kv, head_dim, **extra)
 
 
 @POSITIONS.register("rope_half_split")

@@ -17,7 +17,7 @@ class TensorSpec:
     """One tensor a part needs from the weight file.
 
     `init` says how the random-weights mode fills it: "normal" (N(0, std)),
-    "ones" or "zeros".  `role` says how it is kept in memory: "matrix" tensors
+    "ones", "zeros" or "eye" (the identity matrix).  `role` says how it is kept in memory: "matrix" tensors
     feed matrix products and are held in the compute dtype, "vector" tensors
     (norm scales, biases) are small and held in float32, "table" tensors are
     integer tables kept as int32, "keep" tensors stay as the file stores them.
@@ -37,6 +37,9 @@ class CacheNeed:
     wholly behind the window are given back.
     kind "none": no pages.
     `state_shape`: per-request state of fixed size kept in a slot, or None.
+    `value_dim`: size of a value head where it differs from the key heads' `head_dim` (0: the same).
+    `block_state_shape`: per-request state that the block around the mixer keeps in the same slot (the last
+    token's normalised row, for a token shift), or None; always float32.
     """
     kind: str = "none"
     n_kv_heads: int = 0
@@ -44,10 +47,16 @@ class CacheNeed:
     window: int | None = None
     state_shape: tuple[int, ...] | None = None
     state_dtype: str = "float32"
+    value_dim: int = 0
+    block_state_shape: tuple[int, ...] | None = None
+
+    @property
+    def v_dim(self) -> int:
+        return self.value_dim or self.head_dim
 
     def page_key(self) -> tuple:
         """Layers with equal keys share one group of pages and one block table."""
-        return (self.kind, self.n_kv_heads, self.head_dim, self.window)
+        return (self.kind, self.n_kv_heads, self.head_dim, self.window, self.v_dim)
 
 
 @dataclasses.dataclass(frozen=True)
@@ -80,6 +89,14 @@ class MixerSpec:
     window: int | None = None
     scale: float | None = None    # None = 1/sqrt(head_dim)
     position: PositionSpec | None = None
+    value_dim: int | None = None  # size of a value head (None = head_dim)
+    chunk: int | None = None      # a query sees only keys of its own run of `chunk` positions, counted from 0
+    distance_bias: float | None = None   # b: head h's scores lose 2^(-b (h+1) / n_heads) per position of distance
+    sink: bool = False            # a learned number per head joins the softmax's denominator
+    own_kv: bool = True           # False: no key/value projections; the layer reads the cache it is pointed at
+    gate_cap: float | None = None  # recurrent mixers: the cap on the gates' pre-activations
+    eps: float = 0.0              # mixers with a norm of their own inside
+    tensor_names: tuple[tuple[str, str], ...] = ()   # (part's name, file's name) where a file names tensors otherwise
     options: dict[str, Any] = dataclasses.field(default_factory=dict, hash=False, compare=False)
 
 
@@ -88,7 +105,11 @@ class FeedForwardSpec:
     kind: str                     # "gated_dense", ...
     hidden_size: int
     intermediate_size: int = 0
-    activation: str = "silu"
+    activation: str = "silu"      # "silu", or "capped_swish" with the three numbers below
+    act_alpha: float = 1.0        # g * sigmoid(alpha g)
+    act_limit: float | None = None  # g is cut at +limit, the other branch at +-limit
+    act_up_shift: float = 0.0     # added to the other branch before the product
+    tensor_names: tuple[tuple[str, str], ...] = ()
     options: dict[str, Any] = dataclasses.field(default_factory=dict, hash=False, compare=False)
 
 
@@ -109,6 +130,8 @@ class LayerSpec:
     feed_forward_prefix: str = ""
     mixer_norm_prefix: str = ""
     feed_forward_norm_prefix: str = ""
+    prefix: str = ""              # of the tensors that belong to the block itself (blocks that have any)
+    options: dict[str, Any] = dataclasses.field(default_factory=dict, hash=False, compare=False)   # the block's own constants
 
     def __post_init__(self):
         if self.mixer is None and self.feed_forward is None:

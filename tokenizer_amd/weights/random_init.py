@@ -34,6 +34,9 @@ def random_tensor(name: str, spec: TensorSpec, seed: int, norm_spread: float = 0
             return torch.ones(spec.shape, dtype=torch.bfloat16)
         noise = torch.empty(spec.shape, dtype=torch.float32).normal_(0.0, 1.0, generator=_generator(seed, name))
         return (1.0 + float(norm_spread) * noise).to(torch.bfloat16)
+    if spec.init == "eye":                 # a square mixing matrix: the identity, or near it when a spread is asked for
+        noise = torch.empty(spec.shape, dtype=torch.float32).normal_(0.0, 1.0, generator=_generator(seed, name))
+        return (torch.eye(spec.shape[0], spec.shape[1]) + float(norm_spread) * noise).to(torch.bfloat16)
     if spec.init == "zeros":
         return torch.zeros(spec.shape, dtype=torch.bfloat16)
     if spec.init != "normal":
