@@ -52,6 +52,15 @@ class CachePools:
         return (pages[index, :keys].view(*shape, page_size, need.head_dim),
                 pages[index, keys:].view(*shape, need.v_dim, page_size))
 
+    def keep_states(self) -> list:
+        """Copies of every state tensor (for a run whose effect on them is to be undone)."""
+        return [(t, t.clone()) for t in list(self.states.values()) + list(self.block_states.values())]
+
+    @staticmethod
+    def put_states_back(kept: list) -> None:
+        for tensor, copy in kept:
+            tensor.copy_(copy)
+
     def bytes(self) -> int:
         return sum(t.numel() * t.element_size() for t in self.pages) + \
             sum(t.numel() * t.element_size() for t in list(self.states.values()) + list(self.block_states.values()))

@@ -9,14 +9,18 @@
 // q: rows of `q_stride` elements, head h at h*d.  out: [n_tokens, n_q*d].
 // Token t at position p of entry e sees keys max(0, p-window)..p (window < 0: all from 0), whose
 // pages are block_table[e, key / page_size]; a token of entry -1 is passed over (its output row is not written).  Key pages: [n_pages, n_kv, page_size, d]; value pages
-// are transposed inside a page: [n_pages, n_kv, d, page_size].
+// are transposed inside a page: [n_pages, n_kv, dv, page_size] (dv: the size of a value head; out is [n_tokens, n_q*dv]).
+// chunk > 0: only keys of the query's own run of `chunk` positions (runs counted from position 0) are seen.
+// slopes (float [n_q] or null): head h's score loses slopes[h] for every position between query and key.
+// sinks (float [n_q] or null): exp(sinks[h]) joins the softmax's denominator (no key, no value, not scaled, no bias).
 template <typename T>
 __global__ void __launch_bounds__(ATT_WAVES * WAVE)
 paged_attention_generic(const T* __restrict__ q, int q_stride, T* __restrict__ out,
                         const T* __restrict__ k_pages, const T* __restrict__ v_pages,
                         const int* __restrict__ positions, const int* __restrict__ entry_of_token,
                         const int* __restrict__ block_table, int table_stride,
-                        int n_q, int n_kv, int d, int page_size, int window, float scale) {
+                        int n_q, int n_kv, int d, int page_size, int window, float scale, int dv, int chunk,
+                        const float* __restrict__ slopes, const float* __restrict__ sinks) {
   __shared__ float q_s[ATT_MAX_D];
   __shared__ float acc_s[ATT_WAVES][ATT_MAX_D];
   __shared__ float m_s[ATT_WAVES], l_s[ATT_WAVES];
@@ -28,8 +32,10 @@ paged_attention_generic(const T* __restrict__ q, int q_stride, T* __restrict__ o
   const int pos = positions[t];
   const int* table = block_table + (size_t)entry * table_stride;
   const int kvh = h / (n_q / n_kv);
-  const int lo = (window >= 0 && pos > window) ? pos - window : 0;
+  int lo = (window >= 0 && pos > window) ? pos - window : 0;
+  if (chunk > 0) lo = max(lo, pos / chunk * chunk);
   const int n_keys = pos - lo + 1;
+  const float slope = slopes ? slopes[h] : 0.f;
 
   for (int i = threadIdx.x; i < d; i += blockDim.x) q_s[i] = ld(q + (size_t)t * q_stride + (size_t)h * d + i);
   __syncthreads();
@@ -45,7 +51,7 @@ paged_attention_generic(const T* __restrict__ q, int q_stride, T* __restrict__ o
     if (valid) {
       const int page = table[j / page_size];
       row = (page * n_kv + kvh) * page_size + (j % page_size);
-      vbase = (page * n_kv + kvh) * page_size * d + (j % page_size);
+      vbase = (page * n_kv + kvh) * page_size * dv + (j % page_size);
       const T* kr = k_pages + (size_t)row * d;
       float dot = 0.f;
       if (sizeof(T) == 4 && d % 4 == 0) {
@@ -57,7 +63,7 @@ paged_attention_generic(const T* __restrict__ q, int q_stride, T* __restrict__ o
       } else {
         for (int i = 0; i < d; ++i) dot += q_s[i] * ld(kr + i);
       }
-      s = dot * scale;
+      s = dot * scale - slope * (float)(pos - j);
     }
     const float m_new = fmaxf(m, wave_max(s));
     const float p = valid ? expf(s - m_new) : 0.f;
@@ -78,7 +84,7 @@ paged_attention_generic(const T* __restrict__ q, int q_stride, T* __restrict__ o
         const int off = j % page_size;
         const int run = min(count - jj, page_size - off);
         const float* page_v = reinterpret_cast<const float*>(v_pages) +
-                              ((size_t)table[j / page_size] * n_kv + kvh) * d * page_size + off;
+                              ((size_t)table[j / page_size] * n_kv + kvh) * dv * page_size + off;
         if (off % 4 == 0 && run >= 4) {
           for (int q4 = 0; q4 + 4 <= run; q4 += 4) {
             const float p0 = p_s[wave][jj + q4], p1 = p_s[wave][jj + q4 + 1], p2 = p_s[wave][jj + q4 + 2],
@@ -86,7 +92,7 @@ paged_attention_generic(const T* __restrict__ q, int q_stride, T* __restrict__ o
 #pragma unroll
             for (int r = 0; r < ATT_MAX_D / WAVE; ++r) {
               const int i = lane + r * WAVE;
-              if (i < d) {
+              if (i < dv) {
                 const float4 v4 = *reinterpret_cast<const float4*>(page_v + (size_t)i * page_size + q4);
                 acc[r] = fmaf(p0, v4.x, fmaf(p1, v4.y, fmaf(p2, v4.z, fmaf(p3, v4.w, acc[r]))));
               }
@@ -98,7 +104,7 @@ paged_attention_generic(const T* __restrict__ q, int q_stride, T* __restrict__ o
 #pragma unroll
           for (int r = 0; r < ATT_MAX_D / WAVE; ++r) {
             const int i = lane + r * WAVE;
-            if (i < d) acc[r] += pj * page_v[(size_t)i * page_size];
+            if (i < dv) acc[r] += pj * page_v[(size_t)i * page_size];
           }
           ++jj;
         }
@@ -111,7 +117,7 @@ paged_attention_generic(const T* __restrict__ q, int q_stride, T* __restrict__ o
 #pragma unroll
         for (int r = 0; r < ATT_MAX_D / WAVE; ++r) {
           const int i = lane + r * WAVE;
-          if (i < d) acc[r] += pj * ld(vr + (size_t)i * page_size);
+          if (i < dv) acc[r] += pj * ld(vr + (size_t)i * page_size);
         }
       }
     }
@@ -120,22 +126,23 @@ paged_attention_generic(const T* __restrict__ q, int q_stride, T* __restrict__ o
 #pragma unroll
   for (int r = 0; r < ATT_MAX_D / WAVE; ++r) {
     const int i = lane + r * WAVE;
-    if (i < d) acc_s[wave][i] = acc[r];
+    if (i < dv) acc_s[wave][i] = acc[r];
   }
   if (lane == 0) { m_s[wave] = m; l_s[wave] = l; }
   __syncthreads();
   float big = -INFINITY;
   for (int w = 0; w < ATT_WAVES; ++w) big = fmaxf(big, m_s[w]);
-  float denom = 0.f;
+  if (sinks) big = fmaxf(big, sinks[h]);
+  float denom = sinks ? expf(sinks[h] - big) : 0.f;
   float weights[ATT_WAVES];
   for (int w = 0; w < ATT_WAVES; ++w) {
     weights[w] = (m_s[w] == -INFINITY) ? 0.f : expf(m_s[w] - big);
     denom += l_s[w] * weights[w];
   }
-  for (int i = threadIdx.x; i < d; i += blockDim.x) {
+  for (int i = threadIdx.x; i < dv; i += blockDim.x) {
     float v = 0.f;
     for (int w = 0; w < ATT_WAVES; ++w) v += acc_s[w][i] * weights[w];
-    st(out + (size_t)t * n_q * d + (size_t)h * d + i, v / denom);
+    st(out + (size_t)t * n_q * dv + (size_t)h * dv + i, v / denom);
   }
 }
 
@@ -143,17 +150,21 @@ extern "C" int ta_paged_attention_generic(const void* q, int q_stride, void* out
                                           const void* v_pages, const void* positions, const void* entry_of_token,
                                           const void* block_table, int table_stride, int n_tokens, int n_q,
                                           int n_kv, int d, int page_size, int window, float scale, int dtype,
+                                          int dv, int chunk, const void* slopes, const void* sinks,
                                           hipStream_t stream) {
   if (n_tokens <= 0) return 0;
-  if (d > ATT_MAX_D || d <= 0 || n_kv <= 0 || n_q % n_kv) return -1;
+  if (dv <= 0) dv = d;
+  if (d > ATT_MAX_D || dv > ATT_MAX_D || d <= 0 || n_kv <= 0 || n_q % n_kv) return -1;
   dim3 grid(n_tokens, n_q);
   if (dtype == DT_F32)
     paged_attention_generic<float><<<grid, ATT_WAVES * WAVE, 0, stream>>>((const float*)q, q_stride, (float*)out,
         (const float*)k_pages, (const float*)v_pages, (const int*)positions, (const int*)entry_of_token,
-        (const int*)block_table, table_stride, n_q, n_kv, d, page_size, window, scale);
+        (const int*)block_table, table_stride, n_q, n_kv, d, page_size, window, scale, dv, chunk,
+        (const float*)slopes, (const float*)sinks);
   else
     paged_attention_generic<bf16_t><<<grid, ATT_WAVES * WAVE, 0, stream>>>((const bf16_t*)q, q_stride, (bf16_t*)out,
         (const bf16_t*)k_pages, (const bf16_t*)v_pages, (const int*)positions, (const int*)entry_of_token,
-        (const int*)block_table, table_stride, n_q, n_kv, d, page_size, window, scale);
+        (const int*)block_table, table_stride, n_q, n_kv, d, page_size, window, scale, dv, chunk,
+        (const float*)slopes, (const float*)sinks);
   return LAUNCH_STATUS();
 }

@@ -211,6 +211,20 @@ __global__ void silu_gate_kernel(const T* __restrict__ in, T* __restrict__ out, 
   }
 }
 
+// out[t, j] = g' * sigmoid(alpha g') * (u' + shift) with g' = min(in[t, j], limit), u' = clamp(in[t, inner + j], -limit, limit).
+template <typename T>
+__global__ void capped_gate_kernel(const T* __restrict__ in, T* __restrict__ out, int inner, size_t total, float alpha,
+                                   float limit, float shift) {
+  for (size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x; idx < total;
+       idx += (size_t)gridDim.x * blockDim.x) {
+    const size_t t = idx / inner;
+    const int j = (int)(idx - t * inner);
+    const float g = fminf(ld(in + t * 2 * inner + j), limit);
+    const float u = fminf(fmaxf(ld(in + t * 2 * inner + inner + j), -limit), limit);
+    st(out + idx, g / (1.0f + expf(-alpha * g)) * (u + shift));
+  }
+}
+
 // The same for bfloat16 rows whose length is a multiple of 8: sixteen bytes of gate and of up per thread.
 __global__ void silu_gate_vec_kernel(const bf16_t* __restrict__ in, bf16_t* __restrict__ out, int inner8,
                                      unsigned total8) {
@@ -299,6 +313,18 @@ extern "C" int ta_silu_gate(const void* in, void* out, int n_tokens, int inner, 
     silu_gate_kernel<float><<<blocks, 256, 0, stream>>>((const float*)in, (float*)out, inner, total);
   else
     silu_gate_kernel<bf16_t><<<blocks, 256, 0, stream>>>((const bf16_t*)in, (bf16_t*)out, inner, total);
+  return LAUNCH_STATUS();
+}
+
+extern "C" int ta_capped_gate(const void* in, void* out, int n_tokens, int inner, float alpha, float limit, float shift,
+                              int dtype, hipStream_t stream) {
+  const size_t total = (size_t)n_tokens * inner;
+  if (total == 0) return 0;
+  const int blocks = (int)((total + 255) / 256 < 65535 ? (total + 255) / 256 : 65535);
+  if (dtype == DT_F32)
+    capped_gate_kernel<float><<<blocks, 256, 0, stream>>>((const float*)in, (float*)out, inner, total, alpha, limit, shift);
+  else
+    capped_gate_kernel<bf16_t><<<blocks, 256, 0, stream>>>((const bf16_t*)in, (bf16_t*)out, inner, total, alpha, limit, shift);
   return LAUNCH_STATUS();
 }
 

@@ -12,14 +12,15 @@ template <typename T>
 __global__ void rope_store_kernel(T* __restrict__ qkv, int row_stride, const float* __restrict__ bias,
                                   const int* __restrict__ positions, const float* __restrict__ cos_sin,
                                   const int* __restrict__ slots, T* __restrict__ k_pages, T* __restrict__ v_pages,
-                                  int n_q, int n_kv, int d, int page_size) {
+                                  int n_q, int n_kv, int d, int page_size, int dv) {
   const int t = blockIdx.x;
-  const int head = blockIdx.y;  // 0..n_q-1 q, then n_kv k heads, then n_kv v heads
-  T* x = qkv + (size_t)t * row_stride + (size_t)head * d;
-  const float* b = bias ? bias + (size_t)head * d : nullptr;
-  const int half = d / 2;
+  const int head = blockIdx.y;  // 0..n_q-1 q, then n_kv k heads, then n_kv v heads (of dv elements each)
   const bool is_v = head >= n_q + n_kv;
   const bool is_k = !is_v && head >= n_q;
+  const size_t at = is_v ? (size_t)(n_q + n_kv) * d + (size_t)(head - n_q - n_kv) * dv : (size_t)head * d;
+  T* x = qkv + (size_t)t * row_stride + at;
+  const float* b = bias ? bias + at : nullptr;
+  const int half = d / 2;
   T* dst = nullptr;
   int dst_stride = 1;   // distance between consecutive elements of the head in the page
   if ((is_k || is_v) && slots) {
@@ -27,14 +28,15 @@ __global__ void rope_store_kernel(T* __restrict__ qkv, int row_stride, const flo
     if (slot >= 0) {
       const int page = slot / page_size, off = slot - page * page_size;
       const int kvh = is_k ? head - n_q : head - n_q - n_kv;
-      T* base = (is_k ? k_pages : v_pages) + ((size_t)page * n_kv + kvh) * page_size * d;
+      T* base = (is_k ? k_pages : v_pages) + ((size_t)page * n_kv + kvh) * page_size * (is_k ? d : dv);
       if (is_k) dst = base + (size_t)off * d;
       else { dst = base + off; dst_stride = page_size; }
     }
   }
   if (is_v || !cos_sin) {
     if (!b && !dst) return;
-    for (int i = threadIdx.x; i < d; i += blockDim.x) {
+    const int size = is_v ? dv : d;
+    for (int i = threadIdx.x; i < size; i += blockDim.x) {
       float v = ld(x + i);
       if (b) { v += b[i]; st(x + i, v); }
       if (dst) st(dst + (size_t)i * dst_stride, v);
@@ -154,10 +156,11 @@ rope_store_vec_kernel(bf16_t* __restrict__ qkv, int row_stride, const float* __r
 
 extern "C" int ta_rope_store(void* qkv, int row_stride, const void* bias, const void* positions,
                              const void* cos_sin, const void* slots, void* k_pages, void* v_pages,
-                             int n_tokens, int n_q, int n_kv, int d, int page_size, int dtype,
+                             int n_tokens, int n_q, int n_kv, int d, int page_size, int dtype, int dv,
                              hipStream_t stream) {
   if (n_tokens <= 0) return 0;
-  if (dtype == DT_BF16 && d % 16 == 0 && row_stride % 8 == 0 && (((uintptr_t)bias | (uintptr_t)cos_sin) & 15) == 0) {
+  if (dv <= 0) dv = d;
+  if (dtype == DT_BF16 && dv == d && d % 16 == 0 && row_stride % 8 == 0 && (((uintptr_t)bias | (uintptr_t)cos_sin) & 15) == 0) {
     const long units = (long)n_tokens * ((n_q + n_kv) * (d / 16) + n_kv * (d / 8));
 #define GO(BB, RR) rope_store_vec_kernel<BB, RR><<<(int)((units + 255) / 256), 256, 0, stream>>>( \
         (bf16_t*)qkv, row_stride, (const float*)bias, (const int*)positions, (const float*)cos_sin, \
@@ -170,9 +173,9 @@ extern "C" int ta_rope_store(void* qkv, int row_stride, const void* bias, const 
   dim3 grid(n_tokens, n_q + 2 * n_kv);
   if (dtype == DT_F32)
     rope_store_kernel<float><<<grid, 64, 0, stream>>>((float*)qkv, row_stride, (const float*)bias, (const int*)positions,
-        (const float*)cos_sin, (const int*)slots, (float*)k_pages, (float*)v_pages, n_q, n_kv, d, page_size);
+        (const float*)cos_sin, (const int*)slots, (float*)k_pages, (float*)v_pages, n_q, n_kv, d, page_size, dv);
   else
     rope_store_kernel<bf16_t><<<grid, 64, 0, stream>>>((bf16_t*)qkv, row_stride, (const float*)bias, (const int*)positions,
-        (const float*)cos_sin, (const int*)slots, (bf16_t*)k_pages, (bf16_t*)v_pages, n_q, n_kv, d, page_size);
+        (const float*)cos_sin, (const int*)slots, (bf16_t*)k_pages, (bf16_t*)v_pages, n_q, n_kv, d, page_size, dv);
   return LAUNCH_STATUS();
 }

@@ -89,9 +89,13 @@ class StepGraph:
         try:
             side = torch.cuda.Stream(device=device)
             side.wait_stream(torch.cuda.current_stream(device))
+            # The eager run writes what the replay writes again.  For keys and values that is the same twice; state
+            # that a step moves on (a recurrence's, a token shift's) would move twice, so it is put back.
+            kept = engine.pools.keep_states()
             with torch.cuda.stream(side):           # one eager run first, so that nothing is set up under capture
                 engine.model.decoder.forward(self.ctx, engine.layer_caches)
             torch.cuda.current_stream(device).wait_stream(side)
+            engine.pools.put_states_back(kept)
             torch.cuda.synchronize(device)
             # A plain decode step (one token per request, its logits wanted) may end by turning its own description
             # into the next step's on the device (`Ops.argmax_next_step`): in a run of such steps the host then

@@ -152,7 +152,9 @@ class Ops:
                      "ta_gemm_skinny_bf16_splitk", "ta_gemm_skinny_qkv_rope", "ta_fused_norm_qkv_rope",
                      "ta_fused_norm_gated", "ta_fused_linear_residual", "ta_fused_qkv_rope", "ta_fused_gated",
                      "ta_splitk_reduce", "ta_splitk_add_rmsnorm", "ta_argmax", "ta_argmax_next_step", "ta_sample",
-                     "ta_sample_workspace_words", "ta_library_gemm_bf16", "ta_compute_units", "ta_read_stream"):
+                     "ta_sample_workspace_words", "ta_library_gemm_bf16", "ta_compute_units", "ta_read_stream",
+                     "ta_embedding_streams", "ta_streams_step", "ta_token_shift", "ta_mlstm_scan", "ta_head_norm_gate",
+                     "ta_capped_gate"):
             getattr(self.lib, name).restype = ctypes.c_int
         self.lib.ta_library_gemm_bf16.argtypes = [ctypes.c_void_p] * 4 + [ctypes.c_int] * 5 + [
             ctypes.c_void_p, ctypes.c_size_t, ctypes.c_int, ctypes.c_void_p]
@@ -265,12 +267,19 @@ class Ops:
         return out
 
     # ------------------------------------------------------------- gated activation
-    def silu_gate(self, gate_up: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
-        """out = silu(gate_up[:, :I]) * gate_up[:, I:].  gate_up [T, 2I]; out [T, I]."""
+    def silu_gate(self, gate_up: torch.Tensor, out: torch.Tensor, act: tuple | None = None) -> torch.Tensor:
+        """out = silu(gate_up[:, :I]) * gate_up[:, I:].  gate_up [T, 2I]; out [T, I].  With `act` = (alpha, limit,
+        shift): g' = min(g, limit), u' = clamp(u, -limit, limit), out = g' * sigmoid(alpha g') * (u' + shift)."""
         _dev(gate_up, out)
         n_tokens, two_inner = gate_up.shape
         _need(two_inner % 2 == 0 and tuple(out.shape) == (n_tokens, two_inner // 2) and out.dtype == gate_up.dtype,
               "silu_gate shapes do not fit")
+        if act is not None:
+            alpha, limit, shift = act
+            self._check(self.lib.ta_capped_gate(_ptr(gate_up), _ptr(out), n_tokens, two_inner // 2, ctypes.c_float(alpha),
+                                                ctypes.c_float(limit), ctypes.c_float(shift), _code(out.dtype),
+                                                self._stream()), "capped_gate")
+            return out
         self._check(self.lib.ta_silu_gate(_ptr(gate_up), _ptr(out), n_tokens, two_inner // 2,
                                           _code(out.dtype), self._stream()), "silu_gate")
         return out
@@ -279,18 +288,19 @@ class Ops:
     def rope_store(self, qkv: torch.Tensor, bias: torch.Tensor | None, positions: torch.Tensor,
                    cos_sin: torch.Tensor | None, slots: torch.Tensor | None,
                    k_pages: torch.Tensor | None, v_pages: torch.Tensor | None,
-                   n_q: int, n_kv: int, head_dim: int) -> None:
+                   n_q: int, n_kv: int, head_dim: int, value_dim: int | None = None) -> None:
         """Add bias, rotate q and k heads in place, store k and v heads into their pages.
 
-        qkv [T, (n_q + 2 n_kv) d]; bias float32 or None; positions int32 [T];
+        qkv [T, (n_q + n_kv) d + n_kv dv] (dv = `value_dim`, d if None); bias float32 or None; positions int32 [T];
         cos_sin float32 [P, d] (cos half, sin half) or None for no rotation;
         slots int32 [T] (page * page_size + offset, negative = skip) or None;
         key pages [n_pages, n_kv, page_size, d], value pages [n_pages, n_kv, d, page_size].
         """
         _dev(qkv, bias, positions, cos_sin, slots, k_pages, v_pages)
         n_tokens, width = qkv.shape
-        _need(width == (n_q + 2 * n_kv) * head_dim, "qkv width does not match the head counts")
-        _need(head_dim % 2 == 0, "head size must be even")
+        value_dim = head_dim if value_dim is None else int(value_dim)
+        _need(width == (n_q + n_kv) * head_dim + n_kv * value_dim, "qkv width does not match the head counts")
+        _need(head_dim % 2 == 0 or cos_sin is None, "head size must be even")
         _need(positions.dtype == torch.int32 and positions.numel() == n_tokens, "positions must be int32 [T]")
         page_size = 1
         if bias is not None:
@@ -301,19 +311,21 @@ class Ops:
             _need(slots.dtype == torch.int32 and slots.numel() == n_tokens, "slots must be int32 [T]")
             _need(k_pages is not None and v_pages is not None, "slots without pages")
             _need(k_pages.dtype == qkv.dtype and v_pages.dtype == qkv.dtype, "pages must have the dtype of qkv")
-            page_size = self._page_size(k_pages, v_pages, n_kv, head_dim)
+            page_size = self._page_size(k_pages, v_pages, n_kv, head_dim, value_dim)
         self._check(self.lib.ta_rope_store(_ptr(qkv), width, _ptr(bias), _ptr(positions), _ptr(cos_sin),
                                            _ptr(slots), _ptr(k_pages), _ptr(v_pages), n_tokens, n_q, n_kv,
-                                           head_dim, page_size, _code(qkv.dtype), self._stream()), "rope_store")
+                                           head_dim, page_size, _code(qkv.dtype), value_dim, self._stream()), "rope_store")
 
     @staticmethod
-    def _page_size(k_pages: torch.Tensor, v_pages: torch.Tensor, n_kv: int, head_dim: int) -> int:
+    def _page_size(k_pages: torch.Tensor, v_pages: torch.Tensor, n_kv: int, head_dim: int,
+                   value_dim: int | None = None) -> int:
+        value_dim = head_dim if value_dim is None else value_dim
         _need(k_pages.dim() == 4 and k_pages.shape[1] == n_kv and k_pages.shape[3] == head_dim,
               "key pages must be [n_pages, n_kv, page_size, d]")
         page_size = k_pages.shape[2]
-        _need(tuple(v_pages.shape) == (k_pages.shape[0], n_kv, head_dim, page_size),
-              "value pages must be [n_pages, n_kv, d, page_size]")
-        _need(k_pages.numel() < 2 ** 31, "a layer's pages must hold fewer than 2^31 elements")
+        _need(tuple(v_pages.shape) == (k_pages.shape[0], n_kv, value_dim, page_size),
+              "value pages must be [n_pages, n_kv, dv, page_size]")
+        _need(k_pages.numel() < 2 ** 31 and v_pages.numel() < 2 ** 31, "a layer's pages must hold fewer than 2^31 elements")
         return page_size
 
     # ------------------------------------------------------------------ attention
@@ -321,8 +333,14 @@ class Ops:
                         v_pages: torch.Tensor, positions: torch.Tensor, entry_of_token: torch.Tensor,
                         block_table: torch.Tensor, n_q: int, n_kv: int, head_dim: int,
                         window: int | None, scale: float, max_position: int | None = None,
-                        batch=None) -> torch.Tensor:
+                        batch=None, value_dim: int | None = None, chunk: int | None = None,
+                        slopes: torch.Tensor | None = None, sinks: torch.Tensor | None = None) -> torch.Tensor:
         """Causal attention of every token over the pages of its request.
+
+        Beyond the plain form: `value_dim` (value heads of dv elements; out is [T, n_q dv]), `chunk` (only keys
+        of the query's own run of so many positions, counted from position 0), `slopes` (float32 [n_q]: head h's
+        score loses slopes[h] per position of distance), `sinks` (float32 [n_q]: exp(sinks[h]) joins the
+        denominator).  Scores and weights are float32.
 
         qkv [T, >= n_q d] (query heads first); out [T, n_q d]; key pages [n_pages, n_kv, page_size, d],
         value pages [n_pages, n_kv, d, page_size];
@@ -333,18 +351,24 @@ class Ops:
         """
         _dev(qkv, out, k_pages, v_pages, positions, entry_of_token, block_table)
         n_tokens = qkv.shape[0]
+        value_dim = head_dim if value_dim is None else int(value_dim)
+        _dev(slopes, sinks)
+        for extra in (slopes, sinks):
+            _need(extra is None or (extra.dtype == torch.float32 and extra.numel() == n_q), "slopes and sinks are float32 [n_q]")
+        _need(chunk is None or chunk > 0, "a chunk has at least one position")
+        plain = value_dim == head_dim and chunk is None and slopes is None and sinks is None
         _need(qkv.shape[1] >= n_q * head_dim, "qkv is narrower than the query heads")
-        _need(tuple(out.shape) == (n_tokens, n_q * head_dim) and out.dtype == qkv.dtype, "attention output shape")
+        _need(tuple(out.shape) == (n_tokens, n_q * value_dim) and out.dtype == qkv.dtype, "attention output shape")
         _need(k_pages.dtype == qkv.dtype and v_pages.dtype == qkv.dtype, "pages must have the dtype of qkv")
-        page_size = self._page_size(k_pages, v_pages, n_kv, head_dim)
+        page_size = self._page_size(k_pages, v_pages, n_kv, head_dim, value_dim)
         _need(positions.dtype == torch.int32 and positions.numel() == n_tokens, "positions must be int32 [T]")
         _need(entry_of_token.dtype == torch.int32 and entry_of_token.numel() == n_tokens, "entry_of_token must be int32 [T]")
         _need(block_table.dtype == torch.int32 and block_table.dim() == 2, "block_table must be int32 [E, P]")
         _need(n_kv > 0 and n_q % n_kv == 0, "query heads must be a multiple of kv heads")
-        _need(0 < head_dim <= 256, "head sizes up to 256 are supported")
+        _need(0 < head_dim <= 256 and 0 < value_dim <= 256, "head sizes up to 256 are supported")
         if max_position is not None:
             _need(max_position // page_size < block_table.shape[1], "block table is too narrow for the positions")
-        if (qkv.dtype == torch.bfloat16 and head_dim in self.DECODE_HEAD_DIMS and page_size % 16 == 0
+        if (plain and qkv.dtype == torch.bfloat16 and head_dim in self.DECODE_HEAD_DIMS and page_size % 16 == 0
                 and qkv.shape[1] % 8 == 0 and self.use_fast_attention):
             args = (qkv, out, k_pages, v_pages, positions, entry_of_token, block_table, n_q, n_kv, head_dim,
                     page_size, window, scale, max_position)
@@ -377,7 +401,7 @@ class Ops:
             _ptr(qkv), qkv.shape[1], _ptr(out), _ptr(k_pages), _ptr(v_pages), _ptr(positions),
             _ptr(entry_of_token), _ptr(block_table), block_table.shape[1], n_tokens, n_q, n_kv, head_dim,
             page_size, -1 if window is None else int(window), ctypes.c_float(scale), _code(qkv.dtype),
-            self._stream()), "paged_attention")
+            value_dim, 0 if chunk is None else int(chunk), _ptr(slopes), _ptr(sinks), self._stream()), "paged_attention")
         return out
 
     DECODE_HEAD_DIMS = (16, 32, 48, 64, 80, 96, 112, 128, 160, 192, 224, 256)
@@ -586,8 +610,10 @@ class Ops:
     #                      projection): there the rows' re-reading per tile of 16 columns costs more than tiling
     use_library_gemm = True
 
-    def linear_silu_gate(self, x: torch.Tensor, weight: torch.Tensor, out: torch.Tensor | None = None) -> torch.Tensor:
-        """out = silu(x @ Wg.T) * (x @ Wu.T) for weight = [Wg; Wu] of shape [2I, K]; out [M, I].
+    def linear_silu_gate(self, x: torch.Tensor, weight: torch.Tensor, out: torch.Tensor | None = None,
+                         act: tuple | None = None) -> torch.Tensor:
+        """out = silu(x @ Wg.T) * (x @ Wu.T) for weight = [Wg; Wu] of shape [2I, K]; out [M, I].  `act`: another
+        gated activation than silu (see `silu_gate`).
 
         Few bfloat16 rows run in one kernel; otherwise the product and the gated activation are two."""
         _need(weight.dim() == 2 and weight.shape[0] % 2 == 0, "the joined gate and up matrix has an even row count")
@@ -595,6 +621,8 @@ class Ops:
         if out is None:
             out = torch.empty((m, inner), dtype=x.dtype, device=x.device)
         _need(tuple(out.shape) == (m, inner) and out.dtype == x.dtype and out.is_contiguous(), "gated output shape")
+        if act is not None:
+            return self.silu_gate(self.linear(x, weight), out, act=act)
         if (x.dtype == torch.bfloat16 and m <= self.SKINNY_ROWS
                 and not (self.use_library_gemm and m > self.FUSED_ROWS
                          and weight.shape[0] * weight.shape[1] >= self.GATED_LIBRARY_WEIGHT)):
@@ -723,6 +751,128 @@ class Ops:
             _need(bias.dtype == torch.float32 and bias.numel() == n, "bias must be float32 [N]")
         self._check(self.lib.ta_fused_linear_residual(_ptr(x), lda, _ptr(weight), _ptr(bias), _ptr(residual), m, n, k,
                                                       self.fused_rows, self.fused_waves, self._stream()), "linear_add")
+
+    # ------------------------------------------------------- several residual streams
+    MAX_STREAMS = 8
+
+    def embedding_streams(self, ids: torch.Tensor, table: torch.Tensor, positions: torch.Tensor,
+                          rates: torch.Tensor | None, out: torch.Tensor) -> torch.Tensor:
+        """out[t, s] = table[ids[t]] (+ the position vector of positions[t]: entry 2i sin(p rates[i]), entry 2i+1
+        the cosine) for every stream s.  ids, positions int32 [T]; table [V, W]; rates float32 [W / 2] or None;
+        out float32 [T, S, W]."""
+        _dev(ids, table, positions, rates, out)
+        n, (vocab, width) = ids.numel(), table.shape
+        _need(ids.dtype == torch.int32 and positions.dtype == torch.int32 and positions.numel() == n, "ids, positions int32 [T]")
+        _need(out.dtype == torch.float32 and out.dim() == 3 and out.shape[0] == n and out.shape[2] == width, "out float32 [T, S, W]")
+        if rates is not None:
+            _need(rates.dtype == torch.float32 and width % 2 == 0 and rates.numel() == width // 2, "rates float32 [W / 2]")
+        self._check(self.lib.ta_embedding_streams(_ptr(ids), _ptr(table), _ptr(positions), _ptr(rates), _ptr(out), n, width,
+                                                  vocab, out.shape[1], _code(table.dtype), self._stream()), "embedding_streams")
+        return out
+
+    fuses_single_shift = True     # `streams_step(shift=...)` exists here (steps of one token per request)
+
+    def streams_step(self, streams: torch.Tensor, write, read: torch.Tensor, gain: torch.Tensor, eps: float,
+                     out: torch.Tensor, rows: torch.Tensor | None = None, shift: tuple | None = None) -> torch.Tensor:
+        """Apply a sub-layer's write to the streams and make the next normalised read, in one kernel.
+
+        streams float32 [T, S, W].  `write` (or None): an object with y [T, W], mix float32 [S, S] (indexed [from,
+        to]), out float32 [S], scale float32 [W] or None: x_t <- sum_s mix[s, t] x_s + out[t] * scale * y, stored
+        back unless `rows` (int32 [R]) picks a subset.  Then u = sum_s read[s] x_s and
+        out[i] = u / sqrt(mean(u^2) + eps) * gain[0], out [R or T, W] float32 or the dtype of y.
+        `shift` = (mu float32 [W], state float32 [slots, W], ctx), for steps of one token per request: the row
+        written is h + (state row - h) * mu (zeros for the state at position 0) and h becomes the state row."""
+        _dev(streams, read, gain, out, rows)
+        _need(streams.dtype == torch.float32 and streams.dim() == 3, "streams are float32 [T, S, W]")
+        n_tokens, n_streams, width = streams.shape
+        _need(n_streams <= self.MAX_STREAMS, f"at most {self.MAX_STREAMS} streams")
+        _need(read.dtype == torch.float32 and read.numel() == n_streams and gain.dtype == torch.float32 and gain.numel() == 1,
+              "read float32 [S], gain float32 [1]")
+        n_rows = n_tokens if rows is None else rows.numel()
+        _need(tuple(out.shape) == (n_rows, width), "the read has the wrong shape")
+        if rows is not None:
+            _need(rows.dtype == torch.int32 and shift is None, "rows must be int32 (and no shift over a subset)")
+        y = mix = coef = scale = None
+        y_code = _code(out.dtype)
+        if write is not None:
+            y, mix, coef, scale = write.y, write.mix, write.out, write.scale
+            _dev(y, mix, coef, scale)
+            _need(tuple(y.shape) == (n_tokens, width) and mix.dtype == torch.float32 and tuple(mix.shape) == (n_streams, n_streams)
+                  and coef.dtype == torch.float32 and coef.numel() == n_streams, "the write does not fit the streams")
+            _need(scale is None or (scale.dtype == torch.float32 and scale.numel() == width), "scale float32 [W]")
+            y_code = _code(y.dtype)
+        _need(out.dtype == torch.float32 or _code(out.dtype) == y_code, "the read is float32 or has the dtype of y")
+        mu = state = entry_of_token = state_slots = positions = None
+        if shift is not None:
+            mu, state, ctx = shift
+            entry_of_token, state_slots, positions = ctx.entry_of_token, ctx.state_slots, ctx.positions
+            _dev(mu, state, entry_of_token, state_slots, positions)
+            _need(mu.dtype == torch.float32 and mu.numel() == width and state.dtype == torch.float32 and state.dim() == 2
+                  and state.shape[1] == width, "mu float32 [W], state float32 [slots, W]")
+            _need(entry_of_token.numel() == n_tokens and positions.numel() == n_tokens, "the batch description does not fit")
+        self._check(self.lib.ta_streams_step(_ptr(streams), _ptr(y), _ptr(mix), _ptr(coef), _ptr(scale), _ptr(read), _ptr(gain),
+                                             ctypes.c_float(eps), _ptr(out), _ptr(rows), n_rows, width, n_streams, y_code,
+                                             _code(out.dtype), _ptr(mu), _ptr(state), _ptr(entry_of_token),
+                                             _ptr(state_slots), _ptr(positions), self._stream()), "streams_step")
+        return out
+
+    def token_shift(self, h: torch.Tensor, mu: torch.Tensor, state: torch.Tensor, cu_q: torch.Tensor,
+                    first_position: torch.Tensor, state_slots: torch.Tensor, entry_of_token: torch.Tensor,
+                    out: torch.Tensor) -> torch.Tensor:
+        """out[t] = h[t] + (before - h[t]) * mu, `before` = h[t - 1] within an entry's rows, the entry's state row for
+        its first token (zeros if its first position is 0); the entry's last row of h becomes its state row.
+        h float32 [T, W]; mu float32 [W]; state float32 [slots, W]; cu_q int32 [E + 1]; first_position, state_slots
+        int32 [E]; entry_of_token int32 [T]; out [T, W]."""
+        _dev(h, mu, state, cu_q, first_position, state_slots, entry_of_token, out)
+        n_tokens, width = h.shape
+        _need(h.dtype == torch.float32 and mu.dtype == torch.float32 and mu.numel() == width, "h float32 [T, W], mu float32 [W]")
+        _need(state.dtype == torch.float32 and state.dim() == 2 and state.shape[1] == width, "state float32 [slots, W]")
+        _need(tuple(out.shape) == (n_tokens, width) and entry_of_token.numel() == n_tokens, "token_shift shapes do not fit")
+        _need(first_position.numel() == cu_q.numel() - 1 == state_slots.numel(), "one first position and slot per entry")
+        self._check(self.lib.ta_token_shift(_ptr(h), _ptr(mu), _ptr(state), _ptr(cu_q), _ptr(first_position), _ptr(state_slots),
+                                            _ptr(entry_of_token), _ptr(out), n_tokens, width, _code(out.dtype),
+                                            self._stream()), "token_shift")
+        return out
+
+    # -------------------------------------------------------------- matrix memory
+    def mlstm_scan(self, qkvg: torch.Tensor, gates: torch.Tensor, state: torch.Tensor, cu_q: torch.Tensor,
+                   first_position: torch.Tensor, state_slots: torch.Tensor, out: torch.Tensor,
+                   heads: int, d: int, dv: int, cap: float) -> torch.Tensor:
+        """The matrix-memory recurrence over every entry's rows, from and into the entries' state rows.
+
+        qkvg [T, >= 2 heads d + heads dv]: q, k (heads of d) and v (heads of dv) side by side; gates float32
+        [T, >= 2 heads]: pre-activations of the input and of the forget gate; state float32 [slots, heads d dv +
+        heads d + heads] (C, n, m; an entry whose first position is 0 starts from zeros); out float32 [T, heads dv]."""
+        _dev(qkvg, gates, state, cu_q, first_position, state_slots, out)
+        n_tokens = qkvg.shape[0]
+        _need(qkvg.shape[1] >= 2 * heads * d + heads * dv and 0 < d <= 256, "q, k, v do not fit the rows (d up to 256)")
+        _need(gates.dtype == torch.float32 and gates.shape[0] == n_tokens and gates.shape[1] >= 2 * heads, "gates float32 [T, 2 heads]")
+        _need(state.dtype == torch.float32 and state.dim() == 2 and state.shape[1] >= heads * d * dv + heads * d + heads,
+              "state rows are too short")
+        _need(out.dtype == torch.float32 and tuple(out.shape) == (n_tokens, heads * dv), "out float32 [T, heads dv]")
+        n_entries = cu_q.numel() - 1
+        _need(first_position.numel() == n_entries == state_slots.numel(), "one first position and slot per entry")
+        coef = torch.empty((n_tokens, heads, 3), dtype=torch.float32, device=qkvg.device)
+        self._check(self.lib.ta_mlstm_scan(_ptr(qkvg), qkvg.shape[1], _ptr(gates), gates.shape[1], _ptr(state),
+                                           ctypes.c_long(state.shape[1]), _ptr(cu_q), _ptr(first_position), _ptr(state_slots),
+                                           _ptr(coef), _ptr(out), n_entries, heads, d, dv, ctypes.c_float(cap),
+                                           _code(qkvg.dtype), self._stream()), "mlstm_scan")
+        return out
+
+    def head_norm_gate(self, read: torch.Tensor, weight: torch.Tensor, gate_rows: torch.Tensor, gate_offset: int,
+                       eps: float, heads: int, dv: int, out: torch.Tensor) -> torch.Tensor:
+        """out[t, h] = read[t, h] / sqrt(mean(read[t, h]^2) + eps) * weight[h] * sigmoid(gate[t, h]), heads of dv; the gate
+        lies in `gate_rows` from column `gate_offset` on.  read float32 [T, heads dv]; weight float32 [heads dv]."""
+        _dev(read, weight, gate_rows, out)
+        n_tokens = read.shape[0]
+        _need(read.dtype == torch.float32 and read.shape[1] == heads * dv and weight.dtype == torch.float32
+              and weight.numel() == heads * dv, "read float32 [T, heads dv], weight float32 [heads dv]")
+        _need(gate_rows.shape[0] == n_tokens and gate_rows.shape[1] >= gate_offset + heads * dv and gate_rows.dtype == out.dtype
+              and tuple(out.shape) == (n_tokens, heads * dv), "the gate's rows do not fit")
+        self._check(self.lib.ta_head_norm_gate(_ptr(read), _ptr(weight), _ptr(gate_rows), gate_rows.shape[1], gate_offset,
+                                               ctypes.c_float(eps), n_tokens, heads, dv, _ptr(out), _code(out.dtype),
+                                               self._stream()), "head_norm_gate")
+        return out
 
     # ------------------------------------------------------------------- sampling
     def argmax(self, logits: torch.Tensor, out: torch.Tensor | None = None) -> torch.Tensor:
