@@ -109,7 +109,7 @@ class PlainOps:
                 row = torch.zeros_like(row)
             c = row[:size_c].reshape(heads, d, dv).clone()
             n = row[size_c:size_c + size_n].reshape(heads, d).clone()
-            m = row[size_c + size_n:].clone()
+            m = row[size_c + size_n:size_c + size_n + heads].clone()
             for t in range(lo, hi):
                 q = qkvg[t, :heads * d].to(w).reshape(heads, d) * d ** -0.5
                 k = qkvg[t, heads * d:2 * heads * d].to(w).reshape(heads, d)
@@ -123,7 +123,7 @@ class PlainOps:
                 m = new_m
                 floor = torch.maximum((n * q).sum(-1).abs(), torch.exp(-m)) + 1e-6
                 out[t] = (torch.einsum("hdv,hd->hv", c, q) / floor[:, None]).reshape(-1).to(out.dtype)
-            state[slot] = torch.cat([c.reshape(-1), n.reshape(-1), m]).to(state.dtype)
+            state[slot, :size_c + size_n + heads] = torch.cat([c.reshape(-1), n.reshape(-1), m]).to(state.dtype)
         return out
 
     def head_norm_gate(self, read, weight, gate_rows, gate_offset, eps, heads, dv, out):

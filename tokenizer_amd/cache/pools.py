@@ -66,6 +66,6 @@ class CachePools:
             sum(t.numel() * t.element_size() for t in list(self.states.values()) + list(self.block_states.values()))
 
     def poison(self, value: float = float("nan")) -> None:
-        """Fill every page with a value that shows if a kernel reads what no request wrote."""
-        for tensor in self.pages:
+        """Fill every page and state row with a value that shows if a kernel reads what no request wrote."""
+        for tensor in self.pages + list(self.states.values()) + list(self.block_states.values()):
             tensor.fill_(value)
