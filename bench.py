@@ -17,6 +17,13 @@ share a prefix of 1,024 ids, with the prefix cache) and prints one JSON line for
     python bench.py [--size 0.5b|1.5b|7b] --attention TOKENS [--cached C] [--attention-kernel auto|per-wave|shared]
 
 times the prompt attention kernel alone on a portion of TOKENS tokens after C cached ones.
+
+    python bench.py --design napadra [--size 0.5b|1.5b|7b] [--layers N] [--batch B] [--steps K]
+
+times a prefill of 2,048 tokens and decoding at batch B of a Napadra model whose layers have the sizes of the
+Qwen2.5 model named (width, heads, feed-forward and vocabulary; its layers alternate attention, attention on the
+layer before's keys and values, matrix memory, attention), and of the Qwen2 model itself with the same number of
+layers, side by side, and prints one JSON line.  `--only napadra|qwen2` runs one of the two (for a profile).
 """
 from __future__ import annotations
 
@@ -238,6 +245,59 @@ def run_workload(name: str, layers: int | None, dtype: str, temperature: float =
                               a == b for a, b in zip(*tokens_of_pass))}}
 
 
+def napadra_config(sizes: dict, layers: int, chunk: int = 4096, streams: int = 4) -> dict:
+    """A Napadra configuration with the layer sizes of a Qwen2 one.  The chunk is as long as the bench's contexts,
+    so that both models' attention reads the same keys; the recurrent layers' heads are twice as wide as the
+    attention's, their values twice as wide again (heads * vdim = width)."""
+    width, heads, kv_heads = sizes["hidden_size"], sizes["num_attention_heads"], sizes["num_key_value_heads"]
+    d = width // heads
+    mlp = {"kind": "dense", "ff": sizes["intermediate_size"], "limit": 7.0}
+    out = []
+    for index in range(layers):
+        kind = index % 4
+        if kind == 2:
+            out.append({"type": "mlstm", "mlp": None,
+                        "mixer": {"heads": max(1, heads // 4), "dim": 2 * d, "vdim": 4 * d, "gate_cap": 15.0}})
+            continue
+        mixer = {"heads": heads, "kv_heads": kv_heads, "dim": d, "vdim": d, "scale": d ** -0.5, "mask": {"size": chunk}}
+        if kind == 1:
+            mixer["kv_from"] = index - 1
+        out.append({"type": "attention", "mixer": mixer, "mlp": mlp})
+    return {"architecture": "Napadra", "vocab": sizes["vocab_size"], "width": width, "streams": streams,
+            "residual_mult": 0.7, "norm": {"eps": 1e-6}, "layers": out}
+
+
+def run_design(args, sizes: dict) -> dict:
+    """Prefill and decode throughput of Napadra beside Qwen2 at equal layer sizes and count."""
+    import torch
+    from tokenizer_amd.config import NapadraConfig, Qwen2Config
+    from tokenizer_amd.engine import random_model
+    layers = args.layers or 8
+    steps = min(args.steps, 256)
+    record = {"design": "napadra", "beside": "qwen2", "size": args.size, "layers": layers, "dtype": args.dtype,
+              "prompt_len": PROMPT_LEN, "batch": args.batch, "decode_steps": steps, "data": "synthetic (random weights)"}
+    configs = {"napadra": lambda: NapadraConfig.from_dict(napadra_config(sizes, layers)),
+               "qwen2": lambda: Qwen2Config.from_dict(dict(sizes, num_hidden_layers=layers))}
+    for name, make in configs.items():
+        if args.only and args.only != name:
+            continue
+        log(f"{name}: building random weights ({layers} layers, {args.dtype})")
+        model = random_model(make(), seed=0, dtype=args.dtype, device="cuda:0")
+        seconds = run_prefill(model, repeats=3)
+        elapsed, _ = run_decode(model, args.batch, steps, args.warmup)
+        record[name] = {"prefill_tokens_per_s": round(PROMPT_LEN / seconds, 1), "prefill_ms": round(seconds * 1e3, 3),
+                        "decode_tokens_per_s": round(args.batch * steps / elapsed, 1),
+                        "decode_ms_per_step": round(elapsed / steps * 1e3, 4),
+                        "weight_bytes_per_step": weight_bytes_per_step(model)}
+        log(f"{name}: {record[name]}")
+        del model
+        torch.cuda.empty_cache()
+    if "napadra" in record and "qwen2" in record:
+        record["prefill_ratio"] = round(record["napadra"]["prefill_tokens_per_s"] / record["qwen2"]["prefill_tokens_per_s"], 3)
+        record["decode_ratio"] = round(record["napadra"]["decode_tokens_per_s"] / record["qwen2"]["decode_tokens_per_s"], 3)
+    return record
+
+
 def measure_peaks() -> dict:
     """What this device reaches on the two yardsticks of the rooflines: reading a large buffer once (4 GiB, by a
     library reduction and by the package's own read loop in the access pattern of its weight-streaming kernels;
@@ -329,6 +389,9 @@ def main() -> int:
     parser.add_argument("--layers", type=int, default=None)
     parser.add_argument("--size", default="0.5b", choices=["0.5b", "1.5b", "7b"],
                         help="layer sizes of the decode benchmark (the default is the one the record is for)")
+    parser.add_argument("--design", default=None, choices=["napadra"],
+                        help="time this design beside Qwen2 at equal layer sizes (prefill and decode)")
+    parser.add_argument("--only", default=None, choices=["napadra", "qwen2"], help="with --design: one of the two models")
     parser.add_argument("--peaks", action="store_true", help="measure what the device reaches in HBM reads and bf16 products")
     parser.add_argument("--workload", default=None, choices=["mixed-1.5b", "mixed-0.5b", "prefix-7b"],
                         help="run a serving workload through the scheduler instead of the decode benchmark")
@@ -373,6 +436,9 @@ def main() -> int:
                                       args.prompts_first, args.decode_burst)), flush=True)
         return 0
     sizes = {"0.5b": QWEN2_0_5B, "1.5b": QWEN2_1_5B, "7b": QWEN2_7B}[args.size]
+    if args.design:
+        print(json.dumps(run_design(args, sizes)), flush=True)
+        return 0
     if args.attention:
         print(json.dumps(run_attention(sizes, args.attention, args.cached, args.attention_kernel)), flush=True)
         return 0

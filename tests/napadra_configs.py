@@ -36,6 +36,17 @@ NAPADRA = {
                       _layer("attention", _attention(8, 1, 16, 8, 5, 0.25, kv_from=0)),
                       _layer("mlstm", {"heads": 4, "dim": 24, "vdim": 16, "gate_cap": 12.0}, ff=48, limit=0.4),
                       _layer("attention", _attention(2, 2, 48, 16, 64, 0.1, kv_from=1), ff=32)]}, 21),
+    # Sizes that are no multiples of eight anywhere (the bfloat16 products fill such a K up), three streams.
+    "S": ({"architecture": "Napadra", "vocab": 97, "width": 52, "streams": 3, "residual_mult": 0.9, "norm": {"eps": 2e-6},
+           "layers": [_layer("attention", _attention(3, 3, 12, 14, 11, 0.4), ff=50, limit=1.2),
+                      _layer("mlstm", {"heads": 3, "dim": 12, "vdim": 20, "gate_cap": 7.0}, ff=30, limit=0.8),
+                      _layer("attention", _attention(6, 3, 12, 14, 26, 0.3, kv_from=0))]}, 13),
+    # Key and value heads of one size (the matrix-core attention kernels in bfloat16), chunks that cut tiles of sixteen tokens.
+    "T": ({"architecture": "Napadra", "vocab": 180, "width": 64, "streams": 2, "residual_mult": 0.7, "norm": {"eps": 1e-6},
+           "layers": [_layer("attention", _attention(4, 2, 16, 16, 19, 0.25), ff=48, limit=1.0),
+                      _layer("attention", _attention(4, 2, 16, 16, 23, 0.25, kv_from=0), ff=48, limit=1.0),
+                      _layer("mlstm", {"heads": 2, "dim": 32, "vdim": 32, "gate_cap": 10.0}),
+                      _layer("attention", _attention(2, 1, 64, 64, 40, 0.125), ff=80, limit=3.0)]}, 34),
 }
 
 

@@ -196,11 +196,15 @@ class Batch:
         self.entry_of_token = i32([e for e, (_, n, _) in enumerate(entries) for _ in range(n)])
         self.positions = i32([p + k for p, n, _ in entries for k in range(n)])
         self.n_tokens = int(self.cu_q[-1])
-        self.q_tiles = i32([0, 0] if any(n != 1 for _, n, _ in entries) else []).reshape(-1, 2)
+        tiles = [[e, at] for e, (_, n, _) in enumerate(entries) if n != 1 for at in range(0, n, 16)]
+        self.q_tiles = i32(tiles).reshape(-1, 2)
+        rows = np.cumsum([0] + [n for _, n, _ in entries])
+        self.decode_rows = i32([int(rows[e]) for e, (_, n, _) in enumerate(entries) if n == 1])
+        self.max_position = max(p + n - 1 for p, n, _ in entries)
 
 
 @pytest.mark.parametrize("backend", BACKENDS)
-@pytest.mark.parametrize("width,streams", [(64, 2), (200, 3), (4352, 1), (24, 8)])
+@pytest.mark.parametrize("width,streams", [(64, 2), (200, 3), (4352, 1), (24, 8), (52, 13)])
 def test_streams_step_alone(backend, width, streams):
     from tokenizer_amd.parts.streams import StreamWrite
     ops, device, dtype = ops_for(backend)
@@ -298,8 +302,9 @@ def test_matrix_memory_alone_in_portions(backend, heads, d, dv):
     assert float((torch.cat(got) - want).abs().max()) <= tol * max(1.0, float(want.abs().max()))
 
 
-def _paged(ops, device, dtype, q, k, v, page_size, chunk, slopes, sinks, scale, first_page=3):
-    """Attention of every row of q (positions 0..n-1 of one request) over keys and values laid into pages."""
+def _paged(ops, device, dtype, q, k, v, page_size, chunk, slopes, sinks, scale, first_page=3, as_prompt=False):
+    """Attention of every row of q (positions 0..n-1 of one request) over keys and values laid into pages.
+    `as_prompt`: the rows are described as one portion of a prompt (the kernels for portions then take them)."""
     n, n_q, d = q.shape
     n_kv, dv = k.shape[1], v.shape[2]
     n_pages = first_page + -(-n // page_size) + 1
@@ -314,13 +319,16 @@ def _paged(ops, device, dtype, q, k, v, page_size, chunk, slopes, sinks, scale, 
     f32 = lambda t: None if t is None else t.float().to(device)
     ops.paged_attention(q.reshape(n, -1).to(dtype).to(device).contiguous(), out, k_pages, v_pages, i32(list(range(n))),
                         i32([0] * n), i32([table]), n_q, n_kv, d, None, scale, max_position=n - 1,
+                        batch=Batch([(0, n, 0)], device) if as_prompt else None,
                         value_dim=dv, chunk=chunk, slopes=f32(slopes), sinks=f32(sinks))
     return out.double().cpu().reshape(n, n_q, dv)
 
 
 @pytest.mark.parametrize("backend", BACKENDS)
-@pytest.mark.parametrize("n_q,n_kv,d,dv,chunk", [(4, 2, 16, 24, 20), (3, 3, 32, 32, 33), (8, 1, 16, 8, 7), (2, 1, 80, 48, 300)])
-def test_attention_alone_against_the_plain_function(backend, n_q, n_kv, d, dv, chunk):
+@pytest.mark.parametrize("as_prompt", [False, True])
+@pytest.mark.parametrize("n_q,n_kv,d,dv,chunk", [(4, 2, 16, 24, 20), (3, 3, 32, 32, 33), (8, 1, 16, 8, 7), (2, 1, 80, 48, 300),
+                                                 (4, 1, 64, 64, 21), (34, 2, 128, 128, 50)])
+def test_attention_alone_against_the_plain_function(backend, n_q, n_kv, d, dv, chunk, as_prompt):
     ops, device, dtype = ops_for(backend)
     gen = torch.Generator().manual_seed(n_q + d)
     n, scale = 75, 0.31
@@ -333,17 +341,18 @@ def test_attention_alone_against_the_plain_function(backend, n_q, n_kv, d, dv, c
     w = {"q": q.t(), "sink": sinks, "o": torch.eye(n_q * dv, dtype=torch.float64)}
     want = plain.attention(h, mixer, w, k.reshape(n, n_kv, d).transpose(0, 1), v.reshape(n, n_kv, dv).transpose(0, 1))
     got = _paged(ops, device, dtype, q.reshape(n, n_q, d), k.reshape(n, n_kv, d), v.reshape(n, n_kv, dv), 16, chunk,
-                 plain.distance_slopes(n_q), sinks, scale)
+                 plain.distance_slopes(n_q), sinks, scale, as_prompt=as_prompt)
     tol = 2e-2 if dtype == torch.bfloat16 else 2e-5
     assert float((got.reshape(n, -1) - want).abs().max()) <= tol * float(want.abs().max())
 
 
 @pytest.mark.parametrize("backend", BACKENDS)
-def test_one_key_that_stands_out_is_seen_just_inside_its_chunk_and_not_just_outside(backend):
+@pytest.mark.parametrize("dv,as_prompt", [(8, False), (16, False), (16, True)])
+def test_one_key_that_stands_out_is_seen_just_inside_its_chunk_and_not_just_outside(backend, dv, as_prompt):
     """Every value is zero but one key's, whose score is made to stand far out: the output is that value (times what
     the sink and the bias leave) when the key lies in the query's chunk, and nothing when it lies just before it."""
     ops, device, dtype = ops_for(backend)
-    n, chunk, d, dv = 130, 48, 16, 8
+    n, chunk, d = 130, 48, 16
     for marked in (0, 47, 48, 63, 64, 95, 96, 127):             # chunk edges and page borders
         q = torch.zeros(n, 1, d, dtype=torch.float64)
         k = torch.zeros(n, 1, d, dtype=torch.float64)
@@ -351,7 +360,8 @@ def test_one_key_that_stands_out_is_seen_just_inside_its_chunk_and_not_just_outs
         q[:, 0, 0] = 8.0
         k[marked, 0, 0] = 8.0
         v[marked, 0, :] = 1.0
-        got = _paged(ops, device, dtype, q, k, v, 16, chunk, torch.tensor([0.01]), torch.tensor([0.0]), 1.0)[:, 0, 0]
+        got = _paged(ops, device, dtype, q, k, v, 16, chunk, torch.tensor([0.01]), torch.tensor([0.0]), 1.0,
+                     as_prompt=as_prompt)[:, 0, 0]
         last_seen = (marked // chunk + 1) * chunk - 1
         for query in range(n):
             if marked <= query <= last_seen:

@@ -27,14 +27,18 @@ __device__ __forceinline__ bf16x8 zero8() {
 // Partials: part_o [n_items, n_q, splits, D] (unnormalised), part_ml [n_items, n_q, splits, 2] (max, sum);
 // with splits == 1 the result goes straight to `out` [n_tokens, n_q * D].
 // AHEAD: a wave asks for its next block of keys while it works on the current one (see below).
-template <int D, int DEC_WAVES, bool AHEAD>
+// EXTRA: chunk > 0: only the keys of the token's own run of `chunk` positions (runs counted from position 0) are seen;
+// slopes (float [n_q] or null): head h's score loses slopes[h] per position between token and key; sinks (float [n_q] or
+// null): exp(sinks[h]) joins the softmax's denominator (it rides in the first split's partial sums).
+template <int D, int DEC_WAVES, bool AHEAD, bool EXTRA>
 __global__ void __launch_bounds__(DEC_WAVES * WAVE)
 decode_attention_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_t* __restrict__ out,
                         const bf16_t* __restrict__ k_pages, const bf16_t* __restrict__ vt_pages,
                         const int* __restrict__ rows, const int* __restrict__ positions,
                         const int* __restrict__ entry_of_token, const int* __restrict__ block_table,
                         int table_stride, float* __restrict__ part_o, float* __restrict__ part_ml,
-                        int n_q, int n_kv, int page_size, int window, float scale, int split_keys, int splits) {
+                        int n_q, int n_kv, int page_size, int window, float scale, int split_keys, int splits,
+                        int chunk, const float* __restrict__ slopes, const float* __restrict__ sinks) {
   constexpr int KS = (D + 31) / 32;   // 32-wide steps over the head size for Q K^T
   constexpr int DB = D / 16;          // 16-row blocks of O^T
   HELD(q, q_stride, out, k_pages, vt_pages, rows, positions, entry_of_token, block_table, table_stride, part_o, part_ml,
@@ -60,12 +64,15 @@ decode_attention_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_t* __re
   // An entry past the request's pages may hold anything; it is only used for keys that exist (see load_block).
   const int early_kb = split * split_keys + wave * 32;
   int early_page0 = 0, early_page1 = 0;
-  if (window < 0) {
+  const bool from_zero = window < 0 && !(EXTRA && chunk > 0);      // the first key is key 0 whatever the position
+  if (from_zero) {
     early_page0 = scalar_int(table + min(early_kb / page_size, table_stride - 1));
     early_page1 = scalar_int(table + min((early_kb + 16) / page_size, table_stride - 1));
   }
   const int pos = scalar_int(positions + t);
-  const int lo = (window >= 0 && pos > window) ? pos - window : 0;
+  int lo = (window >= 0 && pos > window) ? pos - window : 0;
+  if (EXTRA && chunk > 0) lo = max(lo, pos / chunk * chunk);
+  const float slope = (EXTRA && slopes && col < heads_here) ? slopes[head] : 0.f;
   const int first = (lo / 32) * 32 + split * split_keys;  // first key of this split (a multiple of 32)
   const int last = min(pos, first + split_keys - 1);
 
@@ -114,7 +121,7 @@ decode_attention_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_t* __re
       // the branch is the same for the whole wave, and the addresses are a page number a lane away from scalars.
       const bool there0 = kb + 15 >= lo, there1 = kb + 16 <= last;
       int page0, page1;
-      if (window < 0 && kb == early_kb) {                    // (without a window the first half always holds keys)
+      if (from_zero && kb == early_kb) {                    // (without a window the first half always holds keys)
         page0 = early_page0;
         page1 = there1 ? early_page1 : early_page0;
       } else {
@@ -167,7 +174,9 @@ decode_attention_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_t* __re
 #pragma unroll
       for (int r = 0; r < 4; ++r) {
         const int key = kb + 8 * g + 4 * t + r;
-        s[t][r] = (blk.active && key >= lo && key <= last) ? st[r] * scale : -INFINITY;
+        float score = st[r] * scale;
+        if (EXTRA) score = fmaf(-slope, (float)(pos - key), score);
+        s[t][r] = (blk.active && key >= lo && key <= last) ? score : -INFINITY;
       }
     }
     float mx = fmaxf(fmaxf(fmaxf(s[0][0], s[0][1]), fmaxf(s[0][2], s[0][3])),
@@ -242,14 +251,19 @@ decode_attention_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_t* __re
     float big = -INFINITY;
 #pragma unroll
     for (int w = 0; w < DEC_WAVES; ++w) big = fmaxf(big, m_s[w][h]);
+    const int hg = kvh * group + hb * 16 + h;
     float o = 0.f, denom = 0.f;
+    if (EXTRA && sinks && split == 0) {
+      const float sink = sinks[hg];
+      big = fmaxf(big, sink);
+      denom = __expf(sink - big);
+    }
 #pragma unroll
     for (int w = 0; w < DEC_WAVES; ++w) {
       const float wgt = (m_s[w][h] == -INFINITY) ? 0.f : __expf(m_s[w][h] - big);
       o += acc_s[w][d][h] * wgt;
       denom += l_s[w][h] * wgt;
     }
-    const int hg = kvh * group + hb * 16 + h;
     if (splits == 1) {
       st(out + (size_t)t * n_q * D + (size_t)hg * D + d, o / denom);
     } else {
@@ -344,15 +358,17 @@ static int launch_decode(const void* q, int q_stride, void* out, const void* k_p
                          const void* rows, const void* positions, const void* entry_of_token,
                          const void* block_table, int table_stride, void* part_o, void* part_ml, int n_items,
                          int n_q, int n_kv, int page_size, int window, float scale, int split_keys, int splits,
-                         hipStream_t stream) {
+                         int chunk, const void* slopes, const void* sinks, hipStream_t stream) {
   const int group = n_q / n_kv;
   dim3 grid(splits, n_kv * ((group + 15) / 16), n_items);
   constexpr int NW = D > 128 ? 2 : 4;   // keeps the merge buffer within 64 KB of LDS
-#define GO(AHEAD) decode_attention_kernel<D, NW, AHEAD><<<grid, NW * WAVE, 0, stream>>>( \
+#define GO(AHEAD, EE) decode_attention_kernel<D, NW, AHEAD, EE><<<grid, NW * WAVE, 0, stream>>>( \
       (const bf16_t*)q, q_stride, (bf16_t*)out, (const bf16_t*)k_pages, (const bf16_t*)vt_pages, (const int*)rows, \
       (const int*)positions, (const int*)entry_of_token, (const int*)block_table, table_stride, (float*)part_o, \
-      (float*)part_ml, n_q, n_kv, page_size, window, scale, split_keys, splits)
-  if (split_keys <= 32 * NW * 8) GO(true); else GO(false);      // up to eight blocks a wave
+      (float*)part_ml, n_q, n_kv, page_size, window, scale, split_keys, splits, chunk, (const float*)slopes, \
+      (const float*)sinks)
+  if (chunk > 0 || slopes || sinks) { if (split_keys <= 32 * NW * 8) GO(true, true); else GO(false, true); }
+  else if (split_keys <= 32 * NW * 8) GO(true, false); else GO(false, false);      // up to eight blocks a wave
 #undef GO
   int status = LAUNCH_STATUS();
   if (status == 0 && splits > 1) {
@@ -382,11 +398,12 @@ extern "C" int ta_decode_attention_bf16(const void* q, int q_stride, void* out, 
                                         const void* entry_of_token, const void* block_table, int table_stride,
                                         void* part_o, void* part_ml, int n_items, int n_q, int n_kv, int d,
                                         int page_size, int window, float scale, int split_keys, int splits,
-                                        hipStream_t stream) {
+                                        int chunk, const void* slopes, const void* sinks, hipStream_t stream) {
   if (n_items <= 0) return 0;
   if (n_kv <= 0 || n_q % n_kv || page_size % 16 || split_keys % 32 || splits < 1) return -1;
 #define CASE(DD) case DD: return launch_decode<DD>(q, q_stride, out, k_pages, vt_pages, rows, positions, entry_of_token, \
-    block_table, table_stride, part_o, part_ml, n_items, n_q, n_kv, page_size, window, scale, split_keys, splits, stream);
+    block_table, table_stride, part_o, part_ml, n_items, n_q, n_kv, page_size, window, scale, split_keys, splits, chunk, \
+    slopes, sinks, stream);
   switch (d) {
     CASE(16) CASE(32) CASE(48) CASE(64) CASE(80) CASE(96) CASE(112) CASE(128) CASE(160) CASE(192) CASE(224) CASE(256)
     default: return -2;

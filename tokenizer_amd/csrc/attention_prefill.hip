@@ -22,11 +22,14 @@ __device__ __forceinline__ bf16x8 pf_zero8() {
 // One step of the online softmax over 64 keys (sixteen consecutive keys lie inside one page) for the HG heads of
 // the wave.  FULL: every key of the block is visible to every token of the tile, so nothing is masked.
 // Scores stay unscaled; `c` = scale * log2(e) enters in exp2(s*c - m*c).
-template <int D, int HG, bool FULL>
+// EXTRA: head h's score (still unscaled) loses `slope[h]` (the head's slope over the scale) per position between the
+// token and the key.
+template <int D, int HG, bool FULL, bool EXTRA>
 __device__ __forceinline__ void prefill_block(
     const bf16_t* __restrict__ k_pages, const bf16_t* __restrict__ vt_pages, const int* __restrict__ table,
     int kb, int kvh, int n_kv, int page_size, int col, int g, int heads_here, int my_pos, int my_lo, int lo, int hi,
-    float c, const bf16x8 (&qf)[HG][(D + 31) / 32], floatx4 (&acc)[HG][D / 16], float (&m)[HG], float (&l)[HG]) {
+    float c, const bf16x8 (&qf)[HG][(D + 31) / 32], floatx4 (&acc)[HG][D / 16], float (&m)[HG], float (&l)[HG],
+    const float (&slope)[HG]) {
   constexpr int KS = (D + 31) / 32;
   constexpr int DB = D / 16;
   // The block is two halves of 32 keys.  Key base + k of a half is index k of the second product's contraction
@@ -106,11 +109,13 @@ __device__ __forceinline__ void prefill_block(
         st = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf[t][ks], qf[h][ks], st, 0, 0, 0);
 #pragma unroll
       for (int r = 0; r < 4; ++r) {
+        const int key = kb + 32 * (t >> 1) + 8 * g + 4 * (t & 1) + r;     // (keys outside lo..hi lie outside my_lo..my_pos)
+        float score = st[r];
+        if (EXTRA) score = fmaf(-slope[h], (float)(my_pos - key), score);
         if (FULL) {
-          s[t * 4 + r] = st[r];
+          s[t * 4 + r] = score;
         } else {
-          const int key = kb + 32 * (t >> 1) + 8 * g + 4 * (t & 1) + r;     // (keys outside lo..hi lie outside my_lo..my_pos)
-          s[t * 4 + r] = (key <= my_pos && key >= my_lo) ? st[r] : -INFINITY;
+          s[t * 4 + r] = (key <= my_pos && key >= my_lo) ? score : -INFINITY;
         }
       }
     }
@@ -150,13 +155,14 @@ __device__ __forceinline__ void prefill_block(
 // tiles: [n_tiles, 2] = (entry, offset of the tile's first token inside the entry's tokens).
 // cu_q[e]: first row of entry e; first_position[e]: position of that row.
 // K pages [n_pages, n_kv, page_size, D]; V^T pages [n_pages, n_kv, D, page_size]; page_size % 16 == 0.
-template <int D, int HG, int NWV>
+template <int D, int HG, int NWV, bool EXTRA>
 __global__ void __launch_bounds__(NWV * WAVE, (D <= 64 && HG <= 2) ? 3 : 1)
 prefill_attention_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_t* __restrict__ out,
                          const bf16_t* __restrict__ k_pages, const bf16_t* __restrict__ vt_pages,
                          const int* __restrict__ tiles, int n_tiles, const int* __restrict__ cu_q,
                          const int* __restrict__ first_position, const int* __restrict__ block_table,
-                         int table_stride, int n_q, int n_kv, int page_size, int window, float scale_log2) {
+                         int table_stride, int n_q, int n_kv, int page_size, int window, float scale_log2,
+                         int chunk, const float* __restrict__ slopes, const float* __restrict__ sinks, float inv_scale) {
   constexpr int KS = (D + 31) / 32;
   constexpr int DB = D / 16;
   HELD(q, q_stride, out, k_pages, vt_pages, tiles, n_tiles, cu_q, first_position, block_table, table_stride, n_q, n_kv,
@@ -191,9 +197,24 @@ prefill_attention_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_t* __r
   const int my_pos = p0 + min(col, n_valid - 1);          // padded columns repeat the last token
   const int my_row = row0 + min(col, n_valid - 1);
   const int hi = p0 + n_valid - 1;                         // last key any token of the tile sees
-  const int lo = (window >= 0 && p0 > window) ? p0 - window : 0;      // first key any token sees
-  const int lo_all = (window >= 0 && hi > window) ? hi - window : 0;  // first key every token sees
-  const int my_lo = (window >= 0 && my_pos > window) ? my_pos - window : 0;
+  int lo = (window >= 0 && p0 > window) ? p0 - window : 0;      // first key any token sees
+  int lo_all = (window >= 0 && hi > window) ? hi - window : 0;  // first key every token sees
+  int my_lo = (window >= 0 && my_pos > window) ? my_pos - window : 0;
+  float slope[HG];
+#pragma unroll
+  for (int h = 0; h < HG; ++h) slope[h] = 0.f;
+  if (EXTRA) {
+    if (chunk > 0) {          // a token sees the keys of its own run of `chunk` positions only; a tile may lie across two runs
+      lo = max(lo, p0 / chunk * chunk);
+      lo_all = max(lo_all, hi / chunk * chunk);
+      my_lo = max(my_lo, my_pos / chunk * chunk);
+    }
+    if (slopes) {
+#pragma unroll
+      for (int h = 0; h < HG; ++h)
+        if (h < heads_here) slope[h] = slopes[head0 + h] * inv_scale;
+    }
+  }
   const int* table = block_table + (size_t)entry * table_stride;
 
   bf16x8 qf[HG][KS];
@@ -221,14 +242,14 @@ prefill_attention_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_t* __r
   // block: in one loop over both, the accumulators would be copied between the variants' registers every turn.
   int kb = (lo / 64) * 64 + 64 * wave;
   for (; kb <= hi && kb < lo_all; kb += 64 * NWV)
-    prefill_block<D, HG, false>(k_pages, vt_pages, table, kb, kvh, n_kv, page_size, col, g, heads_here, my_pos,
-                                my_lo, lo, hi, scale_log2, qf, acc, m, l);
+    prefill_block<D, HG, false, EXTRA>(k_pages, vt_pages, table, kb, kvh, n_kv, page_size, col, g, heads_here, my_pos,
+                                my_lo, lo, hi, scale_log2, qf, acc, m, l, slope);
   for (; kb + 63 <= p0; kb += 64 * NWV)
-    prefill_block<D, HG, true>(k_pages, vt_pages, table, kb, kvh, n_kv, page_size, col, g, heads_here, my_pos,
-                               my_lo, lo, hi, scale_log2, qf, acc, m, l);
+    prefill_block<D, HG, true, EXTRA>(k_pages, vt_pages, table, kb, kvh, n_kv, page_size, col, g, heads_here, my_pos,
+                               my_lo, lo, hi, scale_log2, qf, acc, m, l, slope);
   for (; kb <= hi; kb += 64 * NWV)
-    prefill_block<D, HG, false>(k_pages, vt_pages, table, kb, kvh, n_kv, page_size, col, g, heads_here, my_pos,
-                                my_lo, lo, hi, scale_log2, qf, acc, m, l);
+    prefill_block<D, HG, false, EXTRA>(k_pages, vt_pages, table, kb, kvh, n_kv, page_size, col, g, heads_here, my_pos,
+                                my_lo, lo, hi, scale_log2, qf, acc, m, l, slope);
   if (NWV > 1) {
     // Waves 1.. hand their state to wave 0: maximum, sum and the output accumulators of each head.
     if (wave > 0) {
@@ -270,9 +291,24 @@ prefill_attention_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_t* __r
 #pragma unroll
   for (int h = 0; h < HG; ++h) {
     if (h >= heads_here) break;
+    float sink_term = 0.f;
+    if (EXTRA && sinks) {
+      // exp(sink) joins the denominator: under the larger of the running maximum and the sink, so that neither overflows.
+      const float sink2 = sinks[head0 + h] * 1.4426950408889634f;
+      const float mc = (m[h] == -INFINITY) ? -INFINITY : m[h] * scale_log2;
+      const float top = fmaxf(mc, sink2);
+      const float f = __builtin_amdgcn_exp2f(mc - top);
+      sink_term = __builtin_amdgcn_exp2f(sink2 - top);
+      l[h] *= f;
+#pragma unroll
+      for (int db = 0; db < DB; ++db)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) acc[h][db][r] *= f;
+    }
     float total = l[h];
     total += __shfl_xor(total, 16, WAVE);
     total += __shfl_xor(total, 32, WAVE);
+    total += sink_term;
     if (col >= n_valid) continue;
     const float inv = 1.0f / total;
     bf16_t* dst = out + (size_t)my_row * n_q * D + (size_t)(head0 + h) * D;
@@ -286,18 +322,26 @@ prefill_attention_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_t* __r
   }
 }
 
+struct PrefillExtras {       // what the plain form does not have: see ta_prefill_attention_bf16
+  int chunk;
+  const float* slopes;
+  const float* sinks;
+};
+
 template <int D, int HG, int NWV>
 static int launch_prefill_waves(const void* q, int q_stride, void* out, const void* k_pages, const void* vt_pages,
                                 const void* tiles, int n_tiles, const void* cu_q, const void* first_position,
                                 const void* block_table, int table_stride, int n_q, int n_kv, int page_size,
-                                int window, float scale, hipStream_t stream) {
+                                int window, float scale, PrefillExtras extra, hipStream_t stream) {
   const int group = n_q / n_kv;
   const long workgroups = (long)n_tiles * n_kv * ((group + HG - 1) / HG);
   if (workgroups > 0x7fffffffL) return -1;
-  prefill_attention_kernel<D, HG, NWV><<<(unsigned)workgroups, NWV * WAVE, 0, stream>>>(
-      (const bf16_t*)q, q_stride, (bf16_t*)out, (const bf16_t*)k_pages, (const bf16_t*)vt_pages, (const int*)tiles,
-      n_tiles, (const int*)cu_q, (const int*)first_position, (const int*)block_table, table_stride, n_q, n_kv, page_size,
-      window, scale * 1.4426950408889634f);
+#define GO(EE) prefill_attention_kernel<D, HG, NWV, EE><<<(unsigned)workgroups, NWV * WAVE, 0, stream>>>( \
+      (const bf16_t*)q, q_stride, (bf16_t*)out, (const bf16_t*)k_pages, (const bf16_t*)vt_pages, (const int*)tiles, \
+      n_tiles, (const int*)cu_q, (const int*)first_position, (const int*)block_table, table_stride, n_q, n_kv, page_size, \
+      window, scale * 1.4426950408889634f, extra.chunk, extra.slopes, extra.sinks, 1.0f / scale)
+  if (extra.chunk > 0 || extra.slopes || extra.sinks) GO(true); else GO(false);
+#undef GO
   return LAUNCH_STATUS();
 }
 
@@ -315,9 +359,10 @@ template <int D, int HG>
 static int launch_prefill(const void* q, int q_stride, void* out, const void* k_pages, const void* vt_pages,
                           const void* tiles, int n_tiles, const void* cu_q, const void* first_position,
                           const void* block_table, int table_stride, int n_q, int n_kv, int page_size, int window,
-                          float scale, int max_keys, int waves, hipStream_t stream) {
+                          float scale, int max_keys, int waves, PrefillExtras extra, hipStream_t stream) {
   if (waves == 0) {
-    const int reach = planned_reach(max_keys, window);
+    int reach = planned_reach(max_keys, window);
+    if (extra.chunk > 0 && extra.chunk + 16 < reach) reach = extra.chunk + 16;
     waves = reach > 768 ? 4 : reach > 256 ? 2 : 1;
     // A short portion behind a long cached context: a handful of tiles, each with thousands of keys to walk and a
     // SIMD to itself, so that nothing hides a block's trip to memory.  Eight waves halve each wave's walk (512
@@ -330,7 +375,7 @@ static int launch_prefill(const void* q, int q_stride, void* out, const void* k_
     if (D > 64 && waves > 2) waves = 2;
   }
 #define GO(NWV) launch_prefill_waves<D, HG, NWV>(q, q_stride, out, k_pages, vt_pages, tiles, n_tiles, cu_q, \
-    first_position, block_table, table_stride, n_q, n_kv, page_size, window, scale, stream)
+    first_position, block_table, table_stride, n_q, n_kv, page_size, window, scale, extra, stream)
   if constexpr (D == 48 || D == 64) {          // (the eight waves' states fit the static LDS at these sizes)
     if (waves >= 8) return GO(8);
   }
@@ -377,15 +422,21 @@ extern "C" int ta_prefill_attention_key_splits(int n_tiles, int n_q, int n_kv, i
 // choice).  waves: waves that share a tile's keys in the per-wave kernel (1, 2, 4, 8; 0 = by the reach); asking
 // for a number asks for that kernel.  part_o, part_ml: buffers for `ta_prefill_attention_key_splits(...)` parts of
 // a tile's keys (null: the keys are not cut).
+// chunk > 0: a token sees only the keys of its own run of `chunk` positions (runs counted from position 0); slopes
+// (float [n_q] or null): head h's score loses slopes[h] per position of distance; sinks (float [n_q] or null): exp(sinks[h])
+// joins the softmax's denominator.  With any of the three the per-wave kernel runs, and the keys are not cut.
 extern "C" int ta_prefill_attention_bf16(const void* q, int q_stride, void* out, const void* k_pages,
                                          const void* vt_pages, const void* tiles, int n_tiles, const void* cu_q,
                                          const void* first_position, const void* block_table, int table_stride,
                                          int n_q, int n_kv, int d, int page_size, int window, float scale,
                                          int shared_shape, int max_keys, int waves, int shared,
-                                         void* part_o, void* part_ml, hipStream_t stream) {
+                                         void* part_o, void* part_ml, int chunk, const void* slopes, const void* sinks,
+                                         hipStream_t stream) {
   if (n_tiles <= 0) return 0;
-  if (n_kv <= 0 || n_q % n_kv || page_size % 16) return -1;
-  const int shape = shared_shape_for(n_tiles, n_q, n_kv, d, window, shared_shape, max_keys, waves, shared);
+  if (n_kv <= 0 || n_q % n_kv || page_size % 16 || scale == 0.f) return -1;
+  const PrefillExtras extra = {chunk, (const float*)slopes, (const float*)sinks};
+  const bool plain = chunk <= 0 && !slopes && !sinks;
+  const int shape = plain ? shared_shape_for(n_tiles, n_q, n_kv, d, window, shared_shape, max_keys, waves, shared) : 0;
   if (shape) {
     const int parts = (part_o && part_ml)
         ? ta_prefill_attention_shared_key_splits(n_tiles, n_q, n_kv, planned_reach(max_keys, window), shape) : 1;
@@ -395,7 +446,7 @@ extern "C" int ta_prefill_attention_bf16(const void* q, int q_stride, void* out,
     if (status != -2) return status;
   }
 #define CASE(DD, HG) case DD: return launch_prefill<DD, HG>(q, q_stride, out, k_pages, vt_pages, tiles, n_tiles, cu_q, \
-    first_position, block_table, table_stride, n_q, n_kv, page_size, window, scale, max_keys, waves, stream);
+    first_position, block_table, table_stride, n_q, n_kv, page_size, window, scale, max_keys, waves, extra, stream);
   switch (d) {
     CASE(16, 4) CASE(32, 4) CASE(48, 2) CASE(64, 2) CASE(80, 2) CASE(96, 2) CASE(112, 2) CASE(128, 2)
     CASE(160, 1) CASE(192, 1) CASE(224, 1) CASE(256, 1)

@@ -2,7 +2,7 @@
 // sub-layer's write and makes the next sub-layer's normalised read, and the token shift with its per-request state.
 #include "common.h"
 
-#define MAX_STREAMS 8
+#define MAX_STREAMS 16
 #define KEPT_COLUMNS 16      // columns per thread whose read is kept in registers between the two passes
 
 // out[t, s, :] = table[ids[t], :] (+ the position vector: entry 2i sin(p r_i), entry 2i+1 cos(p r_i)), for every s.
@@ -62,7 +62,7 @@ __device__ __forceinline__ float stream_column(float* __restrict__ x, const TY* 
 // u = sum_s read[s] x_s, h = u / sqrt(mean(u^2) + eps) * gain[0].  With `mu` (one token per request): the row written is
 // h + (before - h) * mu, `before` the state row of the token's request (zeros at position 0), and h becomes the state.
 template <typename TY, typename TO>
-__global__ void __launch_bounds__(256)
+__global__ void __launch_bounds__(1024)
 streams_step_kernel(float* __restrict__ streams, const TY* __restrict__ y, const float* __restrict__ mix,
                     const float* __restrict__ out_coef, const float* __restrict__ scale, const float* __restrict__ read,
                     const float* __restrict__ gain, float eps, TO* __restrict__ out, const int* __restrict__ rows,
@@ -71,9 +71,9 @@ streams_step_kernel(float* __restrict__ streams, const TY* __restrict__ y, const
                     const int* __restrict__ positions) {
   __shared__ float scratch[16];
   __shared__ StreamCoefficients k;
-  if (threadIdx.x < MAX_STREAMS * MAX_STREAMS) {
-    const int s = threadIdx.x / MAX_STREAMS, to = threadIdx.x % MAX_STREAMS;
-    k.mix[threadIdx.x] = (mix && s < S && to < S) ? mix[s * S + to] : 0.f;
+  for (int i = threadIdx.x; i < MAX_STREAMS * MAX_STREAMS; i += blockDim.x) {
+    const int s = i / MAX_STREAMS, to = i % MAX_STREAMS;
+    k.mix[i] = (mix && s < S && to < S) ? mix[s * S + to] : 0.f;
     if (s == 0) {
       k.out[to] = (out_coef && to < S) ? out_coef[to] : 0.f;
       k.read[to] = to < S ? read[to] : 0.f;
@@ -174,7 +174,11 @@ extern "C" int ta_streams_step(void* streams, const void* y, const void* mix, co
   if (n_streams < 1 || n_streams > MAX_STREAMS || width < 1 || !read || !gain || !out) return -1;
   if (y && (!mix || !out_coef)) return -1;
   if (mu && (!state || !entry_of_token || !state_slots || !positions || rows)) return -1;
-#define GO(TY, TO) streams_step_kernel<TY, TO><<<n_rows, 256, 0, stream>>>((float*)streams, (const TY*)y, (const float*)mix, \
+  // Few rows (a decode step): a thread per column, so that a row's loads are one trip to memory instead of one per
+  // 256 columns; many rows fill the device with workgroups of 256.
+  int threads = 256;
+  if (n_rows <= 2 * compute_units()) threads = width >= 1024 ? 1024 : (width + WAVE - 1) / WAVE * WAVE;
+#define GO(TY, TO) streams_step_kernel<TY, TO><<<n_rows, threads, 0, stream>>>((float*)streams, (const TY*)y, (const float*)mix, \
     (const float*)out_coef, (const float*)scale, (const float*)read, (const float*)gain, eps, (TO*)out, (const int*)rows,   \
     width, n_streams, (const float*)mu, (float*)state, (const int*)entry_of_token, (const int*)state_slots,                 \
     (const int*)positions)

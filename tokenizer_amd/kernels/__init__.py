@@ -159,6 +159,7 @@ class Ops:
         self.lib.ta_library_gemm_bf16.argtypes = [ctypes.c_void_p] * 4 + [ctypes.c_int] * 5 + [
             ctypes.c_void_p, ctypes.c_size_t, ctypes.c_int, ctypes.c_void_p]
         self._workspaces: dict[int, torch.Tensor] = {}
+        self._filled: dict[int, tuple] = {}        # weights whose K was filled up to a multiple of eight, by address
         self.compute_units = int(self._loaded.ta_compute_units())     # what the splits below aim to fill
 
     @staticmethod
@@ -368,15 +369,18 @@ class Ops:
         _need(0 < head_dim <= 256 and 0 < value_dim <= 256, "head sizes up to 256 are supported")
         if max_position is not None:
             _need(max_position // page_size < block_table.shape[1], "block table is too narrow for the positions")
-        if (plain and qkv.dtype == torch.bfloat16 and head_dim in self.DECODE_HEAD_DIMS and page_size % 16 == 0
+        # The matrix-core kernels take chunks, slopes and sinks as they are; value heads of another size than the key
+        # heads go to the generic kernel.
+        if (value_dim == head_dim and qkv.dtype == torch.bfloat16 and head_dim in self.DECODE_HEAD_DIMS and page_size % 16 == 0
                 and qkv.shape[1] % 8 == 0 and self.use_fast_attention):
             args = (qkv, out, k_pages, v_pages, positions, entry_of_token, block_table, n_q, n_kv, head_dim,
                     page_size, window, scale, max_position)
+            extras = {} if plain else dict(chunk=chunk, slopes=slopes, sinks=sinks)
             if batch is None:
-                return self._decode_attention(*args)
+                return self._decode_attention(*args, **extras)
             if batch.q_tiles.numel() == 0:
                 # One token per request: request e is row e, the kernel needs no entry-of-token lookup.
-                return self._decode_attention(*args, identity_entries=batch.n_tokens == block_table.shape[0])
+                return self._decode_attention(*args, identity_entries=batch.n_tokens == block_table.shape[0], **extras)
             _need(batch.n_tokens == n_tokens and batch.cu_q.numel() == block_table.shape[0] + 1,
                   "the batch description does not belong to these tokens")
             n_tiles, choice = batch.q_tiles.shape[0], (
@@ -384,7 +388,8 @@ class Ops:
                 self.prefill_waves, self.prefill_shared)
             # A few tiles behind a long context: the launcher cuts each tile's keys over workgroups, whose states
             # a second kernel merges; it says into how many parts, and gets the buffers for them.
-            parts = self.lib.ta_prefill_attention_key_splits(n_tiles, n_q, n_kv, head_dim, *choice) if self.prefill_key_splits else 1
+            parts = self.lib.ta_prefill_attention_key_splits(n_tiles, n_q, n_kv, head_dim, *choice) \
+                if self.prefill_key_splits and plain else 1
             part_o = part_ml = None
             if parts > 1:
                 part_o = torch.empty((n_tiles * 16, n_q, parts, head_dim), dtype=torch.float32, device=qkv.device)
@@ -393,9 +398,10 @@ class Ops:
                 _ptr(qkv), qkv.shape[1], _ptr(out), _ptr(k_pages), _ptr(v_pages), _ptr(batch.q_tiles),
                 n_tiles, _ptr(batch.cu_q), _ptr(batch.first_position), _ptr(block_table),
                 block_table.shape[1], n_q, n_kv, head_dim, page_size, choice[0], ctypes.c_float(scale), *choice[1:],
-                _ptr(part_o), _ptr(part_ml), self._stream()), "prefill_attention")
+                _ptr(part_o), _ptr(part_ml), 0 if chunk is None else int(chunk), _ptr(slopes), _ptr(sinks),
+                self._stream()), "prefill_attention")
             if batch.decode_rows.numel():
-                self._decode_attention(*args, rows=batch.decode_rows)
+                self._decode_attention(*args, rows=batch.decode_rows, **extras)
             return out
         self._check(self.lib.ta_paged_attention_generic(
             _ptr(qkv), qkv.shape[1], _ptr(out), _ptr(k_pages), _ptr(v_pages), _ptr(positions),
@@ -419,7 +425,7 @@ class Ops:
 
     def _decode_attention(self, qkv, out, k_pages, v_pages, positions, entry_of_token, block_table,
                           n_q, n_kv, head_dim, page_size, window, scale, max_position, rows=None,
-                          identity_entries=False):
+                          identity_entries=False, chunk=None, slopes=None, sinks=None):
         """Matrix-core attention of single tokens with the key range split over workgroups."""
         n_items = qkv.shape[0] if rows is None else rows.numel()
         max_keys = (block_table.shape[1] * page_size) if max_position is None else max_position + 1
@@ -428,6 +434,8 @@ class Ops:
         max_keys = -(-max_keys // self.PLAN_KEYS) * self.PLAN_KEYS
         if window is not None:
             max_keys = min(max_keys, window + 32)
+        if chunk is not None:
+            max_keys = min(max_keys, chunk + 32)
         head_blocks = -(-(n_q // n_kv) // 16)
         per_split = max(1, self.target_workgroups // max(1, n_items * n_kv * head_blocks))
         split_keys = max(self.min_split_keys, -(-max_keys // per_split))
@@ -442,7 +450,8 @@ class Ops:
             _ptr(None if identity_entries and rows is None else entry_of_token), _ptr(block_table),
             block_table.shape[1], _ptr(part_o), _ptr(part_ml), n_items,
             n_q, n_kv, head_dim, page_size, -1 if window is None else int(window), ctypes.c_float(scale),
-            split_keys, splits, self._stream()), "decode_attention")
+            split_keys, splits, 0 if chunk is None else int(chunk), _ptr(slopes), _ptr(sinks), self._stream()),
+            "decode_attention")
         return out
 
     # --------------------------------------------------------------------- linear
@@ -480,7 +489,15 @@ class Ops:
                                           self._stream())
         else:
             _need(x.dtype == torch.bfloat16, "linear takes float32 or bfloat16")
-            _need(k % 8 == 0 and lda % 8 == 0, "bfloat16 products need K and the row stride to be multiples of 8")
+            if k % 8 or lda % 8 or x.data_ptr() % 16:
+                # The matrix-core kernels read K sixteen bytes at a time.  A K that is no multiple of eight is filled
+                # up with zeros (the weight once, kept; the rows each time): the sums gain only zeros.
+                fill = (-k) % 8
+                x = torch.nn.functional.pad(x, (0, fill)) if fill or lda % 8 or x.data_ptr() % 16 else x
+                x = x.contiguous()
+                weight = self._filled_weight(weight, fill) if fill else weight
+                m, k = x.shape
+                lda = k
             _need(x.data_ptr() % 16 == 0 and weight.data_ptr() % 16 == 0, "operands must be 16-byte aligned")
             streaming_splits = self._streaming_splits(m, n, k, pending)
             if streaming_splits > 1 and self.split_k_kind == "streaming":
@@ -543,6 +560,14 @@ class Ops:
                                                _code(out_dtype), self._stream())
         self._check(status, "linear")
         return out
+
+    def _filled_weight(self, weight: torch.Tensor, fill: int) -> torch.Tensor:
+        """`weight` with `fill` zero columns behind its K, made once per weight tensor and kept."""
+        kept = self._filled.get(weight.data_ptr())
+        if kept is None or kept[0] is not weight:
+            kept = (weight, torch.nn.functional.pad(weight, (0, fill)).contiguous())
+            self._filled[weight.data_ptr()] = kept
+        return kept[1]
 
     use_split_k = True
     skinny_column_blocks = 0   # blocks of sixteen output columns per workgroup of the weight-streaming kernel: 0 = its choice
@@ -753,7 +778,7 @@ class Ops:
                                                       self.fused_rows, self.fused_waves, self._stream()), "linear_add")
 
     # ------------------------------------------------------- several residual streams
-    MAX_STREAMS = 8
+    MAX_STREAMS = 16
 
     def embedding_streams(self, ids: torch.Tensor, table: torch.Tensor, positions: torch.Tensor,
                           rates: torch.Tensor | None, out: torch.Tensor) -> torch.Tensor:
