@@ -8,16 +8,22 @@
 __device__ __forceinline__ float capped(float z, float cap) { return cap * tanhf(z / cap); }
 __device__ __forceinline__ float log_sigmoid(float z) { return z >= 0.f ? -log1pf(expf(-z)) : z - log1pf(expf(z)); }
 
+#define ML_GROUP 16          // tokens whose q, k (and v) are brought into LDS in one trip
+
 // Pass 1, one wave per (portion, head): token by token the log gates i = cap(gi), f = logsigmoid(cap(gf)), the maximum
 // m' = max(f + m, i), keep = exp(f + m - m'), take = exp(i - m'), n' = keep n + take k, and the divisor
 // max(|n' . q|, exp(-m')) + 1e-6 with q scaled by 1/sqrt(d).  coef[t, h] = (keep, take, divisor); n and m go back into
 // the state.  A portion that starts at position 0 starts from zeros, whatever the slot holds.
+// Tokens are taken sixteen at a time: their q and k rows go into LDS in one trip (the next sixteen are asked for
+// before the current ones are worked on), their gates are worked out side by side in sixteen lanes, and only the
+// recurrence itself walks them one by one.
 template <typename T>
 __global__ void __launch_bounds__(WAVE)
 mlstm_gates_kernel(const T* __restrict__ qkvg, int row_stride, const float* __restrict__ gates, int gate_stride,
                    float* __restrict__ state, size_t state_stride, const int* __restrict__ cu_q,
                    const int* __restrict__ first_position, const int* __restrict__ state_slots,
                    float* __restrict__ coef, int heads, int d, int dv, float cap) {
+  __shared__ float q_s[ML_GROUP][ML_MAX_D], k_s[ML_GROUP][ML_MAX_D];
   const int e = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
   const int lo = cu_q[e], hi = cu_q[e + 1];
   if (hi <= lo) return;                                      // an entry that only fills the batch up
@@ -33,27 +39,62 @@ mlstm_gates_kernel(const T* __restrict__ qkvg, int row_stride, const float* __re
   }
   float m = fresh ? 0.f : *m_state;
   const float q_scale = 1.0f / sqrtf((float)d);
-  for (int t = lo; t < hi; ++t) {
-    const T* x = qkvg + (size_t)t * row_stride;
-    const float i = capped(gates[(size_t)t * gate_stride + h], cap);
-    const float f = log_sigmoid(capped(gates[(size_t)t * gate_stride + heads + h], cap));
-    const float m_new = fmaxf(f + m, i);
-    const float keep = expf(f + m - m_new), take = expf(i - m_new);
-    float dot = 0.f;
+  // Lane l brings elements l, l + 64, ... of the group's 16 * d numbers of q and of k (PIECES of each at most).
+  constexpr int PIECES = ML_GROUP * ML_MAX_D / WAVE;
+  const int pieces = (ML_GROUP * d + WAVE - 1) / WAVE;
+  float q_next[PIECES], k_next[PIECES];
+  auto fetch = [&](int t0) {
 #pragma unroll
-    for (int r = 0; r < ML_MAX_D / WAVE; ++r) {
-      const int j = lane + r * WAVE;
-      if (j < d) {
-        const float q = ld(x + (size_t)h * d + j) * q_scale, k = ld(x + (size_t)(heads + h) * d + j);
-        n[r] = fmaf(keep, n[r], take * k);
-        dot = fmaf(n[r], q, dot);
+    for (int p = 0; p < PIECES; ++p) {
+      if (p >= pieces) break;
+      const int idx = lane + p * WAVE, tok = idx / d, j = idx - tok * d;
+      q_next[p] = k_next[p] = 0.f;
+      if (tok < ML_GROUP && t0 + tok < hi) {
+        const T* x = qkvg + (size_t)(t0 + tok) * row_stride;
+        q_next[p] = ld(x + (size_t)h * d + j) * q_scale;
+        k_next[p] = ld(x + (size_t)(heads + h) * d + j);
       }
     }
-    dot = wave_sum(dot);
-    m = m_new;
-    if (lane == 0) {
-      float* c = coef + ((size_t)t * heads + h) * 3;
-      c[0] = keep; c[1] = take; c[2] = fmaxf(fabsf(dot), expf(-m)) + 1e-6f;
+  };
+  fetch(lo);
+  for (int t0 = lo; t0 < hi; t0 += ML_GROUP) {
+    __syncthreads();
+#pragma unroll
+    for (int p = 0; p < PIECES; ++p) {
+      if (p >= pieces) break;
+      const int idx = lane + p * WAVE, tok = idx / d, j = idx - tok * d;
+      if (tok < ML_GROUP) { q_s[tok][j] = q_next[p]; k_s[tok][j] = k_next[p]; }
+    }
+    // The gates of the group's tokens, one token a lane.
+    float gi = 0.f, gf = 0.f;
+    if (lane < ML_GROUP && t0 + lane < hi) {
+      gi = capped(gates[(size_t)(t0 + lane) * gate_stride + h], cap);
+      gf = log_sigmoid(capped(gates[(size_t)(t0 + lane) * gate_stride + heads + h], cap));
+    }
+    if (t0 + ML_GROUP < hi) fetch(t0 + ML_GROUP);
+    __syncthreads();
+    const int count = min(ML_GROUP, hi - t0);
+    float keep_mine = 0.f, take_mine = 0.f, divisor_mine = 1.f;       // lane l keeps token l's three numbers
+    for (int tok = 0; tok < count; ++tok) {
+      const float i = __shfl(gi, tok, WAVE), f = __shfl(gf, tok, WAVE);
+      const float m_new = fmaxf(f + m, i);
+      const float keep = expf(f + m - m_new), take = expf(i - m_new);
+      float dot = 0.f;
+#pragma unroll
+      for (int r = 0; r < ML_MAX_D / WAVE; ++r) {
+        const int j = lane + r * WAVE;
+        if (j < d) {
+          n[r] = fmaf(keep, n[r], take * k_s[tok][j]);
+          dot = fmaf(n[r], q_s[tok][j], dot);
+        }
+      }
+      dot = wave_sum(dot);
+      m = m_new;
+      if (lane == tok) { keep_mine = keep; take_mine = take; divisor_mine = fmaxf(fabsf(dot), expf(-m)) + 1e-6f; }
+    }
+    if (lane < count) {
+      float* c = coef + ((size_t)(t0 + lane) * heads + h) * 3;
+      c[0] = keep_mine; c[1] = take_mine; c[2] = divisor_mine;
     }
   }
 #pragma unroll
@@ -64,75 +105,93 @@ mlstm_gates_kernel(const T* __restrict__ qkvg, int row_stride, const float* __re
   if (lane == 0) *m_state = m;
 }
 
-// Pass 2, one workgroup of four waves per (portion, head, 64 columns of C): wave w keeps rows w, w + 4, ... of its
-// columns in registers (PER rows a lane), C' = keep C + take k v^T, o = C'^T q / divisor, token by token; the four
-// waves' parts of o are added through LDS.  Columns of C do not depend on each other, so workgroups share nothing.
-// q and k of the next token are fetched while the current one is worked on.
+// Pass 2, one workgroup of four waves per (portion, head, 64 columns of C).  A wave owns sixteen columns; its lanes are
+// (part p = lane / 16, column): lane (p, c) keeps rows p PER .. p PER + PER - 1 of column c in registers, so that
+// C' = keep C + take k v^T and the sum over the rows for o = C'^T q / divisor need no more than two exchanges between
+// lanes per token.  Columns of C do not depend on each other, so waves and workgroups share nothing but the rows of q, k
+// and v, which come into LDS sixteen tokens at a time (the next sixteen are asked for before the current ones are worked on).
 template <typename T, int PER>
 __global__ void __launch_bounds__(4 * WAVE)
 mlstm_memory_kernel(const T* __restrict__ qkvg, int row_stride, const float* __restrict__ coef,
                     float* __restrict__ state, size_t state_stride, const int* __restrict__ cu_q,
                     const int* __restrict__ first_position, const int* __restrict__ state_slots,
                     float* __restrict__ out, int heads, int d, int dv) {
-  __shared__ float qk[2][2][ML_MAX_D];       // [token parity][q, k][d]
-  __shared__ float part[2][4][WAVE];
-  const int e = blockIdx.x, h = blockIdx.y, lane = threadIdx.x & (WAVE - 1), wave = threadIdx.x / WAVE;
+  __shared__ float q_s[ML_GROUP][4 * PER], k_s[ML_GROUP][4 * PER], v_s[ML_GROUP][WAVE], c_s[ML_GROUP][4];
+  const int e = blockIdx.x, h = blockIdx.y, tid = threadIdx.x, lane = tid & (WAVE - 1), wave = tid / WAVE;
   const int lo = cu_q[e], hi = cu_q[e + 1];
   if (hi <= lo) return;
-  const int c = blockIdx.z * WAVE + lane;
+  const int part = lane >> 4, local = wave * 16 + (lane & 15);
+  const int c = blockIdx.z * WAVE + local;
   const bool live = c < dv;
   float* mem = state + (size_t)state_slots[e] * state_stride + (size_t)h * d * dv;
   const bool fresh = first_position[e] == 0;
   float C[PER];
 #pragma unroll
   for (int r = 0; r < PER; ++r) {
-    const int j = wave + 4 * r;
+    const int j = part * PER + r;
     C[r] = (!fresh && live && j < d) ? mem[(size_t)j * dv + c] : 0.f;
   }
   const float q_scale = 1.0f / sqrtf((float)d);
-  const int tid = threadIdx.x;
-  // (Thread i brings q[i] and k[i]: d is at most 256, the workgroup's size.)
-  float q_next = 0.f, k_next = 0.f;
-  if (tid < d) {
-    const T* x = qkvg + (size_t)lo * row_stride;
-    q_next = ld(x + (size_t)h * d + tid) * q_scale;
-    k_next = ld(x + (size_t)(heads + h) * d + tid);
-  }
-  qk[lo & 1][0][tid] = q_next;
-  qk[lo & 1][1][tid] = k_next;
-  __syncthreads();
-  for (int t = lo; t < hi; ++t) {
-    const int now = t & 1;
-    if (t + 1 < hi && tid < d) {
-      const T* x = qkvg + (size_t)(t + 1) * row_stride;
-      q_next = ld(x + (size_t)h * d + tid) * q_scale;
-      k_next = ld(x + (size_t)(heads + h) * d + tid);
-    }
-    const float* cf = coef + ((size_t)t * heads + h) * 3;
-    const float keep = cf[0], take = cf[1], divisor = cf[2];
-    const float v = live ? ld(qkvg + (size_t)t * row_stride + (size_t)2 * heads * d + (size_t)h * dv + c) : 0.f;
-    const float tv = take * v;
-    float acc = 0.f;
+  // Thread i brings elements i, i + 256, ... of the group's 16 * 4 PER numbers of q and of k, and four of the 16 * 64 of v.
+  constexpr int PIECES = ML_GROUP * 4 * PER / (4 * WAVE);
+  float q_next[PIECES], k_next[PIECES], v_next[4], c_next = 0.f;
+  auto fetch = [&](int t0) {
 #pragma unroll
-    for (int r = 0; r < PER; ++r) {
-      const int j = wave + 4 * r;
-      if (j < d) {
-        C[r] = fmaf(keep, C[r], qk[now][1][j] * tv);
-        acc = fmaf(C[r], qk[now][0][j], acc);
+    for (int p = 0; p < PIECES; ++p) {
+      const int idx = tid + p * 4 * WAVE, tok = idx / (4 * PER), j = idx - tok * (4 * PER);
+      q_next[p] = k_next[p] = 0.f;
+      if (j < d && t0 + tok < hi) {
+        const T* x = qkvg + (size_t)(t0 + tok) * row_stride;
+        q_next[p] = ld(x + (size_t)h * d + j) * q_scale;
+        k_next[p] = ld(x + (size_t)(heads + h) * d + j);
       }
     }
-    part[now][wave][lane] = acc;
-    qk[now ^ 1][0][tid] = q_next;
-    qk[now ^ 1][1][tid] = k_next;
+#pragma unroll
+    for (int p = 0; p < 4; ++p) {
+      const int idx = tid + p * 4 * WAVE, tok = idx / WAVE, col = blockIdx.z * WAVE + (idx & (WAVE - 1));
+      v_next[p] = (col < dv && t0 + tok < hi)
+          ? ld(qkvg + (size_t)(t0 + tok) * row_stride + (size_t)2 * heads * d + (size_t)h * dv + col) : 0.f;
+    }
+    if (tid < ML_GROUP * 3) {
+      const int tok = tid / 3;
+      c_next = t0 + tok < hi ? coef[((size_t)(t0 + tok) * heads + h) * 3 + (tid - tok * 3)] : 1.f;
+    }
+  };
+  fetch(lo);
+  for (int t0 = lo; t0 < hi; t0 += ML_GROUP) {
+    __syncthreads();                                         // the group before has been worked off
+#pragma unroll
+    for (int p = 0; p < PIECES; ++p) {
+      const int idx = tid + p * 4 * WAVE, tok = idx / (4 * PER), j = idx - tok * (4 * PER);
+      q_s[tok][j] = q_next[p];
+      k_s[tok][j] = k_next[p];
+    }
+#pragma unroll
+    for (int p = 0; p < 4; ++p) {
+      const int idx = tid + p * 4 * WAVE;
+      v_s[idx / WAVE][idx & (WAVE - 1)] = v_next[p];
+    }
+    if (tid < ML_GROUP * 3) c_s[tid / 3][tid % 3] = c_next;
+    if (t0 + ML_GROUP < hi) fetch(t0 + ML_GROUP);
     __syncthreads();
-    if (wave == 0 && live) {
-      const float sum = (part[now][0][lane] + part[now][1][lane]) + (part[now][2][lane] + part[now][3][lane]);
-      out[(size_t)t * heads * dv + (size_t)h * dv + c] = sum / divisor;
+    const int count = min(ML_GROUP, hi - t0);
+    for (int tok = 0; tok < count; ++tok) {
+      const float keep = c_s[tok][0], tv = c_s[tok][1] * v_s[tok][local];
+      float acc = 0.f;
+#pragma unroll
+      for (int r = 0; r < PER; ++r) {
+        // (Rows past d hold zeros in q and k: they stay zero and add nothing.)
+        C[r] = fmaf(keep, C[r], k_s[tok][part * PER + r] * tv);
+        acc = fmaf(C[r], q_s[tok][part * PER + r], acc);
+      }
+      acc += __shfl_xor(acc, 16, WAVE);
+      acc += __shfl_xor(acc, 32, WAVE);
+      if (part == 0 && live) out[(size_t)(t0 + tok) * heads * dv + (size_t)h * dv + c] = acc / c_s[tok][2];
     }
   }
 #pragma unroll
   for (int r = 0; r < PER; ++r) {
-    const int j = wave + 4 * r;
+    const int j = part * PER + r;
     if (live && j < d) mem[(size_t)j * dv + c] = C[r];
   }
 }
