@@ -10,20 +10,39 @@ __device__ __forceinline__ float log_sigmoid(float z) { return z >= 0.f ? -log1p
 
 #define ML_GROUP 16          // tokens whose q, k (and v) are brought into LDS in one trip
 
+// Lane `from`'s value of v, the same for every lane (`from` is known when the kernel is compiled).
+__device__ __forceinline__ float lane_value(float v, int from) {
+  return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), from));
+}
+
+// x summed over the sixteen lanes of a row (lanes 16 i .. 16 i + 15), in every lane of the row: four rotations within the
+// row, which cost no trip through LDS.
+__device__ __forceinline__ float row_sum16(float x) {
+#define ML_ROR(n) __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(x), 0x120 | (n), 0xF, 0xF, false))
+  x += ML_ROR(8);
+  x += ML_ROR(4);
+  x += ML_ROR(2);
+  x += ML_ROR(1);
+#undef ML_ROR
+  return x;
+}
+
 // Pass 1, one workgroup per (portion, head): token by token the log gates i = cap(gi), f = logsigmoid(cap(gf)), the
 // maximum m' = max(f + m, i), keep = exp(f + m - m'), take = exp(i - m'), n' = keep n + take k, and the divisor
 // max(|n' . q|, exp(-m')) + 1e-6 with q scaled by 1/sqrt(d).  coef[t, h] = (keep, take, divisor); n and m go back into
 // the state.  A portion that starts at position 0 starts from zeros, whatever the slot holds.
-// Tokens are taken sixteen at a time: all four waves bring their q and k rows into LDS in one trip (thread j brings
-// column j; the next sixteen are asked for before the current ones are worked on), the gates are worked out side by
-// side in sixteen lanes, and the first wave walks the recurrence itself token by token.
+// Thread j owns column j of n (d is at most the workgroup's 256 threads).  Tokens are taken sixteen at a time: thread j
+// brings column j of their q and k rows (the next sixteen are asked for before the current ones are worked on); every
+// wave works out the sixteen tokens' gates side by side in sixteen lanes and walks the maximum's chain; the sums
+// n' . q over the columns are made for all sixteen tokens together (within rows of sixteen lanes by rotations, the
+// sixteen rows' sums through LDS).
 template <typename T>
 __global__ void __launch_bounds__(4 * WAVE)
 mlstm_gates_kernel(const T* __restrict__ qkvg, int row_stride, const float* __restrict__ gates, int gate_stride,
                    float* __restrict__ state, size_t state_stride, const int* __restrict__ cu_q,
                    const int* __restrict__ first_position, const int* __restrict__ state_slots,
                    float* __restrict__ coef, int heads, int d, int dv, float cap) {
-  __shared__ float q_s[ML_GROUP][ML_MAX_D], k_s[ML_GROUP][ML_MAX_D];
+  __shared__ float rows_s[ML_GROUP][16];                    // a token's sixteen row sums
   const int e = blockIdx.x, h = blockIdx.y, tid = threadIdx.x, lane = tid & (WAVE - 1), wave = tid / WAVE;
   const int lo = cu_q[e], hi = cu_q[e + 1];
   if (hi <= lo) return;                                      // an entry that only fills the batch up
@@ -31,15 +50,10 @@ mlstm_gates_kernel(const T* __restrict__ qkvg, int row_stride, const float* __re
   float* n_state = row + (size_t)heads * d * dv + (size_t)h * d;
   float* m_state = row + (size_t)heads * d * dv + (size_t)heads * d + h;
   const bool fresh = first_position[e] == 0;
-  float n[ML_MAX_D / WAVE];
-#pragma unroll
-  for (int r = 0; r < ML_MAX_D / WAVE; ++r) {
-    const int j = lane + r * WAVE;
-    n[r] = (wave == 0 && !fresh && j < d) ? n_state[j] : 0.f;
-  }
+  float n = (!fresh && tid < d) ? n_state[tid] : 0.f;
   float m = fresh ? 0.f : *m_state;
   const float q_scale = 1.0f / sqrtf((float)d);
-  float q_next[ML_GROUP], k_next[ML_GROUP];
+  float q_now[ML_GROUP], k_now[ML_GROUP], q_next[ML_GROUP], k_next[ML_GROUP];
   auto fetch = [&](int t0) {
 #pragma unroll
     for (int tok = 0; tok < ML_GROUP; ++tok) {
@@ -53,66 +67,72 @@ mlstm_gates_kernel(const T* __restrict__ qkvg, int row_stride, const float* __re
   };
   fetch(lo);
   for (int t0 = lo; t0 < hi; t0 += ML_GROUP) {
-    __syncthreads();                                         // the group before has been worked off
 #pragma unroll
-    for (int tok = 0; tok < ML_GROUP; ++tok) { q_s[tok][tid] = q_next[tok]; k_s[tok][tid] = k_next[tok]; }
-    // The gates of the group's tokens, one token a lane.
-    float gi = 0.f, gf = 0.f;
-    if (wave == 0 && lane < ML_GROUP && t0 + lane < hi) {
+    for (int tok = 0; tok < ML_GROUP; ++tok) { q_now[tok] = q_next[tok]; k_now[tok] = k_next[tok]; }
+    // The gates of the group's tokens, one token a lane.  A token past the portion's end changes nothing: its forget
+    // gate is 0 (keep 1) and its input gate minus infinity (take 0).
+    float gi = -INFINITY, gf = 0.f;
+    if (lane < ML_GROUP && t0 + lane < hi) {
       gi = capped(gates[(size_t)(t0 + lane) * gate_stride + h], cap);
       gf = log_sigmoid(capped(gates[(size_t)(t0 + lane) * gate_stride + heads + h], cap));
     }
     if (t0 + ML_GROUP < hi) fetch(t0 + ML_GROUP);
-    __syncthreads();
-    if (wave != 0) continue;
-    const int count = min(ML_GROUP, hi - t0);
-    float keep_mine = 0.f, take_mine = 0.f, divisor_mine = 1.f;       // lane l keeps token l's three numbers
-    for (int tok = 0; tok < count; ++tok) {
-      const float i = __shfl(gi, tok, WAVE), f = __shfl(gf, tok, WAVE);
+    // The maximum's chain over the sixteen tokens (three operations a token); lane l keeps what token l needs of it.
+    float m_before = 0.f, m_after = 0.f;
+#pragma unroll
+    for (int tok = 0; tok < ML_GROUP; ++tok) {
+      const float i = lane_value(gi, tok), f = lane_value(gf, tok);
       const float m_new = fmaxf(f + m, i);
-      const float keep = expf(f + m - m_new), take = expf(i - m_new);
+      if (lane == tok) { m_before = m; m_after = m_new; }
+      m = m_new;
+    }
+    // Decays and the divisor's floor of all sixteen tokens side by side.
+    const float keep_mine = expf(gf + m_before - m_after), take_mine = expf(gi - m_after), floor_mine = expf(-m_after);
+    // n' = keep n + take k token by token, and this column's share of n' . q.
+    float share[ML_GROUP];
+#pragma unroll
+    for (int tok = 0; tok < ML_GROUP; ++tok) {
+      n = fmaf(lane_value(keep_mine, tok), n, lane_value(take_mine, tok) * k_now[tok]);
+      share[tok] = n * q_now[tok];
+    }
+#pragma unroll
+    for (int tok = 0; tok < ML_GROUP; ++tok) share[tok] = row_sum16(share[tok]);
+    __syncthreads();                                         // the group before has been read
+    if ((lane & 15) == 0) {
+#pragma unroll
+      for (int tok = 0; tok < ML_GROUP; ++tok) rows_s[tok][tid >> 4] = share[tok];
+    }
+    __syncthreads();
+    if (wave == 0 && lane < ML_GROUP && t0 + lane < hi) {
       float dot = 0.f;
 #pragma unroll
-      for (int r = 0; r < ML_MAX_D / WAVE; ++r) {
-        const int j = lane + r * WAVE;               // (columns past d hold zeros in LDS)
-        n[r] = fmaf(keep, n[r], take * k_s[tok][j]);
-        dot = fmaf(n[r], q_s[tok][j], dot);
-      }
-      dot = wave_sum(dot);
-      m = m_new;
-      if (lane == tok) { keep_mine = keep; take_mine = take; divisor_mine = fmaxf(fabsf(dot), expf(-m)) + 1e-6f; }
-    }
-    if (lane < count) {
+      for (int r = 0; r < 16; ++r) dot += rows_s[lane][r];
       float* c = coef + ((size_t)(t0 + lane) * heads + h) * 3;
-      c[0] = keep_mine; c[1] = take_mine; c[2] = divisor_mine;
+      c[0] = keep_mine; c[1] = take_mine; c[2] = fmaxf(fabsf(dot), floor_mine) + 1e-6f;
     }
   }
-  if (wave != 0) return;
-#pragma unroll
-  for (int r = 0; r < ML_MAX_D / WAVE; ++r) {
-    const int j = lane + r * WAVE;
-    if (j < d) n_state[j] = n[r];
-  }
-  if (lane == 0) *m_state = m;
+  if (tid < d) n_state[tid] = n;
+  if (tid == 0) *m_state = m;
 }
 
 // Pass 2, one workgroup of four waves per (portion, head, 16 columns of C).  A wave owns four columns; its lanes are
-// (part p = lane / 4, column): lane (p, c) keeps rows p, p + 16, p + 32, ... of column c in registers (PER of them), so
-// that C' = keep C + take k v^T and the sum over the rows for o = C'^T q / divisor need four exchanges between lanes per
-// token and nothing else.  Columns of C do not depend on each other, so waves and workgroups share nothing but the rows
-// of q, k and v, which come into LDS sixteen tokens at a time (thread j brings column j of q and of k; the next
-// sixteen are asked for before the current ones are worked on).
+// (column, part p = lane % 16): lane (c, p) keeps rows p PER .. p PER + PER - 1 of column c in registers, so that
+// C' = keep C + take k v^T needs nothing from other lanes and the sum over the rows for o = C'^T q / divisor is a sum
+// within a row of sixteen lanes (four rotations, no trip through LDS).  Columns of C do not depend on each other, so
+// waves and workgroups share nothing but the rows of q, k and v, which come into LDS sixteen tokens at a time (thread
+// j brings column j of q and of k; the next sixteen are asked for before the current ones are worked on).
 template <typename T, int PER>
 __global__ void __launch_bounds__(4 * WAVE)
 mlstm_memory_kernel(const T* __restrict__ qkvg, int row_stride, const float* __restrict__ coef,
                     float* __restrict__ state, size_t state_stride, const int* __restrict__ cu_q,
                     const int* __restrict__ first_position, const int* __restrict__ state_slots,
                     float* __restrict__ out, int heads, int d, int dv) {
-  __shared__ float q_s[ML_GROUP][ML_MAX_D], k_s[ML_GROUP][ML_MAX_D], v_s[ML_GROUP][16], c_s[ML_GROUP][4];
+  __shared__ __attribute__((aligned(16))) float q_s[ML_GROUP][16 * PER], k_s[ML_GROUP][16 * PER];
+  __shared__ float v_s[ML_GROUP][16], c_s[ML_GROUP][4];
   const int e = blockIdx.x, h = blockIdx.y, tid = threadIdx.x, lane = tid & (WAVE - 1), wave = tid / WAVE;
   const int lo = cu_q[e], hi = cu_q[e + 1];
   if (hi <= lo) return;
-  const int part = lane >> 2, local = wave * 4 + (lane & 3);
+  const int part = lane & 15, local = wave * 4 + (lane >> 4);
   const int c = blockIdx.z * 16 + local;
   const bool live = c < dv;
   float* mem = state + (size_t)state_slots[e] * state_stride + (size_t)h * d * dv;
@@ -120,10 +140,12 @@ mlstm_memory_kernel(const T* __restrict__ qkvg, int row_stride, const float* __r
   float C[PER];
 #pragma unroll
   for (int r = 0; r < PER; ++r) {
-    const int j = part + 16 * r;
+    const int j = part * PER + r;
     C[r] = (!fresh && live && j < d) ? mem[(size_t)j * dv + c] : 0.f;
   }
   const float q_scale = 1.0f / sqrtf((float)d);
+  constexpr int PIECES = (16 * PER + 4 * WAVE - 1) / (4 * WAVE);      // columns of q (and of k) a thread brings: 1 here
+  static_assert(PIECES == 1, "a thread brings one column");
   float q_next[ML_GROUP], k_next[ML_GROUP], v_next = 0.f, c_next = 1.f;
   auto fetch = [&](int t0) {
 #pragma unroll
@@ -148,32 +170,52 @@ mlstm_memory_kernel(const T* __restrict__ qkvg, int row_stride, const float* __r
   fetch(lo);
   for (int t0 = lo; t0 < hi; t0 += ML_GROUP) {
     __syncthreads();                                         // the group before has been worked off
+    if (tid < 16 * PER) {
 #pragma unroll
-    for (int tok = 0; tok < ML_GROUP; ++tok) { q_s[tok][tid] = q_next[tok]; k_s[tok][tid] = k_next[tok]; }
+      for (int tok = 0; tok < ML_GROUP; ++tok) { q_s[tok][tid] = q_next[tok]; k_s[tok][tid] = k_next[tok]; }
+    }
     v_s[tid >> 4][tid & 15] = v_next;
     if (tid < ML_GROUP * 3) c_s[tid / 3][tid % 3] = c_next;
     if (t0 + ML_GROUP < hi) fetch(t0 + ML_GROUP);
     __syncthreads();
-    const int count = min(ML_GROUP, hi - t0);
-    for (int tok = 0; tok < count; ++tok) {
+    // Token by token C' = keep C + take k v^T and each lane's share of C'^T q; the sums over a column's sixteen lanes are
+    // made afterwards for all sixteen tokens.  (A token past the portion's end has keep 1 and zeros for k and v: it
+    // changes nothing.  Rows past d hold zeros in q and k: they stay zero and add nothing.)
+    float share[ML_GROUP];
+#pragma unroll
+    for (int tok = 0; tok < ML_GROUP; ++tok) {
       const float keep = c_s[tok][0], tv = c_s[tok][1] * v_s[tok][local];
       float acc = 0.f;
+      if constexpr (PER % 4 == 0) {
 #pragma unroll
-      for (int r = 0; r < PER; ++r) {
-        // (Rows past d hold zeros in q and k: they stay zero and add nothing.)
-        C[r] = fmaf(keep, C[r], k_s[tok][part + 16 * r] * tv);
-        acc = fmaf(C[r], q_s[tok][part + 16 * r], acc);
+        for (int r = 0; r < PER; r += 4) {
+          const float4 k4 = *reinterpret_cast<const float4*>(&k_s[tok][part * PER + r]);
+          const float4 q4 = *reinterpret_cast<const float4*>(&q_s[tok][part * PER + r]);
+          C[r] = fmaf(keep, C[r], k4.x * tv);         acc = fmaf(C[r], q4.x, acc);
+          C[r + 1] = fmaf(keep, C[r + 1], k4.y * tv); acc = fmaf(C[r + 1], q4.y, acc);
+          C[r + 2] = fmaf(keep, C[r + 2], k4.z * tv); acc = fmaf(C[r + 2], q4.z, acc);
+          C[r + 3] = fmaf(keep, C[r + 3], k4.w * tv); acc = fmaf(C[r + 3], q4.w, acc);
+        }
+      } else {
+#pragma unroll
+        for (int r = 0; r < PER; ++r) {
+          C[r] = fmaf(keep, C[r], k_s[tok][part * PER + r] * tv);
+          acc = fmaf(C[r], q_s[tok][part * PER + r], acc);
+        }
       }
-      acc += __shfl_xor(acc, 4, WAVE);
-      acc += __shfl_xor(acc, 8, WAVE);
-      acc += __shfl_xor(acc, 16, WAVE);
-      acc += __shfl_xor(acc, 32, WAVE);
-      if (part == 0 && live) out[(size_t)(t0 + tok) * heads * dv + (size_t)h * dv + c] = acc / c_s[tok][2];
+      share[tok] = acc;
+    }
+#pragma unroll
+    for (int tok = 0; tok < ML_GROUP; ++tok) share[tok] = row_sum16(share[tok]);
+    if (part == 0 && live) {
+#pragma unroll
+      for (int tok = 0; tok < ML_GROUP; ++tok)
+        if (t0 + tok < hi) out[(size_t)(t0 + tok) * heads * dv + (size_t)h * dv + c] = share[tok] / c_s[tok][2];
     }
   }
 #pragma unroll
   for (int r = 0; r < PER; ++r) {
-    const int j = part + 16 * r;
+    const int j = part * PER + r;
     if (live && j < d) mem[(size_t)j * dv + c] = C[r];
   }
 }
