@@ -171,6 +171,19 @@ def test_greedy_generation_through_the_entry_point_and_the_scheduler(folders, ba
         assert sum(a == w for a, w in zip(sum(alone, []), sum(want, []))) >= 20
 
 
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_the_replay_program_on_a_model_folder(folders, oracle, tmp_path, dtype):
+    """bin/trace_run as a child process: the class is chosen by config.json, the pool is made for the trace's peak,
+    four state slots serve ten requests."""
+    name = "T"
+    reqs = requests_for(name, (33, 97, 21, 64, 50, 80, 12, 45, 3, 70))
+    steps = tt.mixed(reqs, 11, max_live=4, tail=14)
+    got = tt.run_program(folders[name], dtype, steps, str(tmp_path / "out"), tt.peak_tokens(steps), NAPADRA[name][0]["vocab"])
+    for rid, ids in reqs.items():
+        close(got[rid], oracle(name, ids), "gpu-" + dtype, rid)
+
+
 # ------------------------------------------------------------------ mechanisms alone
 def ops_for(backend):
     if backend == "cpu":
@@ -326,12 +339,17 @@ def _paged(ops, device, dtype, q, k, v, page_size, chunk, slopes, sinks, scale, 
 
 @pytest.mark.parametrize("backend", BACKENDS)
 @pytest.mark.parametrize("as_prompt", [False, True])
-@pytest.mark.parametrize("n_q,n_kv,d,dv,chunk", [(4, 2, 16, 24, 20), (3, 3, 32, 32, 33), (8, 1, 16, 8, 7), (2, 1, 80, 48, 300),
-                                                 (4, 1, 64, 64, 21), (34, 2, 128, 128, 50)])
-def test_attention_alone_against_the_plain_function(backend, n_q, n_kv, d, dv, chunk, as_prompt):
+@pytest.mark.parametrize("n_q,n_kv,d,dv,chunk,n", [(4, 2, 16, 24, 20, 75), (3, 3, 32, 32, 33, 75), (8, 1, 16, 8, 7, 75),
+                                                   (2, 1, 80, 48, 300, 75), (4, 1, 64, 64, 21, 75), (34, 2, 128, 128, 50, 75),
+                                                   (4, 2, 64, 64, 512, 700)])
+def test_attention_alone_against_the_plain_function(backend, n_q, n_kv, d, dv, chunk, n, as_prompt):
+    """(The last case is long enough for the single-token kernel to cut a token's keys over workgroups, with the sink in
+    the first part's sums, and for several waves to share a tile's keys in the kernel for portions.)"""
     ops, device, dtype = ops_for(backend)
+    if backend == "cpu" and n > 100:
+        pytest.skip("the plain ops walk token by token: the long case is for the kernels")
     gen = torch.Generator().manual_seed(n_q + d)
-    n, scale = 75, 0.31
+    scale = 0.31
     h = torch.eye(n, dtype=torch.float64)                        # so that the projections' weights are q, k, v themselves
     q = rounded(torch.randn(n, n_q * d, generator=gen, dtype=torch.float64), dtype)
     k = rounded(torch.randn(n, n_kv * d, generator=gen, dtype=torch.float64), dtype)

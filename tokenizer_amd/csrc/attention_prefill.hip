@@ -286,6 +286,7 @@ prefill_attention_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_t* __r
 #pragma unroll
           for (int r = 0; r < 4; ++r) acc[h][db][r] += f * merge[w][h][db * 4 + r][lane];
       }
+      m[h] = m_all;                                          // what the sums stand under now (the sink below asks)
     }
   }
 #pragma unroll
