@@ -47,6 +47,12 @@ NAPADRA = {
                       _layer("attention", _attention(4, 2, 16, 16, 23, 0.25, kv_from=0), ff=48, limit=1.0),
                       _layer("mlstm", {"heads": 2, "dim": 32, "vdim": 32, "gate_cap": 10.0}),
                       _layer("attention", _attention(2, 1, 64, 64, 40, 0.125), ff=80, limit=3.0)]}, 34),
+    # Chunks of hundreds of positions: several waves share a tile's keys, single tokens' keys are cut over workgroups.
+    "U": ({"architecture": "Napadra", "vocab": 260, "width": 128, "streams": 2, "residual_mult": 0.6, "norm": {"eps": 1e-6},
+           "layers": [_layer("attention", _attention(4, 2, 32, 32, 300, 0.18), ff=96, limit=1.5),
+                      _layer("mlstm", {"heads": 2, "dim": 64, "vdim": 64, "gate_cap": 15.0}),
+                      _layer("attention", _attention(4, 2, 32, 32, 1024, 0.18, kv_from=0), ff=96, limit=1.5),
+                      _layer("attention", _attention(2, 2, 64, 64, 520, 0.125))]}, 55),
 }
 
 

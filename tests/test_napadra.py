@@ -173,6 +173,19 @@ def test_greedy_generation_through_the_entry_point_and_the_scheduler(folders, ba
 
 @pytest.mark.gpu
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("cut", ["whole", "tail", "portions", "mixed"])
+def test_hundreds_of_tokens_with_long_chunks(folders, oracle, dtype, cut):
+    """Contexts of up to 900 tokens under chunks of 300, 520 and 1,024: keys far back inside a chunk, chunk edges deep in a
+    prompt and among decoded tokens, the decayed memory of hundreds of tokens."""
+    name = "U"
+    reqs = {f"r{i}": random_ids(NAPADRA[name][0]["vocab"], n, 70 + i) for i, n in enumerate((900, 333, 610, 545))}
+    steps = {"whole": lambda: tt.whole(reqs), "tail": lambda: tt.decode_tail(reqs, 48),
+             "portions": lambda: tt.portions(reqs, 9), "mixed": lambda: tt.mixed(reqs, 12, max_live=3, tail=30)}[cut]()
+    check_trace(folders, oracle, name, "gpu-" + dtype, steps, reqs)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_the_replay_program_on_a_model_folder(folders, oracle, tmp_path, dtype):
     """bin/trace_run as a child process: the class is chosen by config.json, the pool is made for the trace's peak,
     four state slots serve ten requests."""
