@@ -32,27 +32,30 @@ struct StreamCoefficients {
 };
 
 // One column of one token: the streams after the write (x' = M^T x + c * g * y), stored if asked, and the read r . x'.
-template <typename TY>
+// SMAX: a bound on S known when the kernel is compiled (4, 8 or 16), so that the loops over the streams unroll to the
+// streams there are.
+template <typename TY, int SMAX>
 __device__ __forceinline__ float stream_column(float* __restrict__ x, const TY* __restrict__ y, const float* __restrict__ scale,
                                                const StreamCoefficients& k, int S, int width, int c, bool store) {
-  float old[MAX_STREAMS], u = 0.f;
+  float old[SMAX], u = 0.f;
 #pragma unroll
-  for (int s = 0; s < MAX_STREAMS; ++s) old[s] = s < S ? x[(size_t)s * width + c] : 0.f;
+  for (int s = 0; s < SMAX; ++s) old[s] = s < S ? x[(size_t)s * width + c] : 0.f;
   if (!y) {
 #pragma unroll
-    for (int s = 0; s < MAX_STREAMS; ++s) if (s < S) u = fmaf(k.read[s], old[s], u);
+    for (int s = 0; s < SMAX; ++s) if (s < S) u = fmaf(k.read[s], old[s], u);
     return u;
   }
   const float add = ld(y + c) * (scale ? scale[c] : 1.0f);
 #pragma unroll
-  for (int to = 0; to < MAX_STREAMS; ++to) {
-    if (to >= S) break;
-    float v = 0.f;
+  for (int to = 0; to < SMAX; ++to) {
+    if (to < S) {
+      float v = 0.f;
 #pragma unroll
-    for (int s = 0; s < MAX_STREAMS; ++s) if (s < S) v = fmaf(k.mix[s * MAX_STREAMS + to], old[s], v);
-    v = fmaf(k.out[to], add, v);
-    if (store) x[(size_t)to * width + c] = v;
-    u = fmaf(k.read[to], v, u);
+      for (int s = 0; s < SMAX; ++s) if (s < S) v = fmaf(k.mix[s * MAX_STREAMS + to], old[s], v);
+      v = fmaf(k.out[to], add, v);
+      if (store) x[(size_t)to * width + c] = v;
+      u = fmaf(k.read[to], v, u);
+    }
   }
   return u;
 }
@@ -61,7 +64,7 @@ __device__ __forceinline__ float stream_column(float* __restrict__ x, const TY* 
 // null; y null = no write) is applied to token r's streams (stored back unless `rows` picks a subset), then
 // u = sum_s read[s] x_s, h = u / sqrt(mean(u^2) + eps) * gain[0].  With `mu` (one token per request): the row written is
 // h + (before - h) * mu, `before` the state row of the token's request (zeros at position 0), and h becomes the state.
-template <typename TY, typename TO>
+template <typename TY, typename TO, int SMAX>
 __global__ void __launch_bounds__(1024)
 streams_step_kernel(float* __restrict__ streams, const TY* __restrict__ y, const float* __restrict__ mix,
                     const float* __restrict__ out_coef, const float* __restrict__ scale, const float* __restrict__ read,
@@ -79,16 +82,66 @@ streams_step_kernel(float* __restrict__ streams, const TY* __restrict__ y, const
       k.read[to] = to < S ? read[to] : 0.f;
     }
   }
-  __syncthreads();
   const int i = blockIdx.x;
   const int r = rows ? rows[i] : i;
   float* x = streams + (size_t)r * S * width;
   const TY* yr = y ? y + (size_t)r * width : nullptr;
   const bool store = y && !rows;
+  if (width <= (int)blockDim.x) {
+    // A thread per column (the launch of a step with few rows): everything the thread needs, the token's slot and
+    // state row too, is asked for before anything is waited for, so the kernel is two trips to memory (the
+    // coefficients and the rows; then the sum over the workgroup) where column after column it was five.
+    const int c = threadIdx.x;
+    const bool in = c < width;
+    int slot = -1;
+    bool first = false;
+    if (mu) {
+      const int e = entry_of_token[r];
+      if (e >= 0) { slot = state_slots[e]; first = positions[r] == 0; }
+    }
+    float old[SMAX];
+#pragma unroll
+    for (int s = 0; s < SMAX; ++s) old[s] = (s < S && in) ? x[(size_t)s * width + c] : 0.f;
+    const float add = (y && in) ? ld(yr + c) * (scale ? scale[c] : 1.0f) : 0.f;
+    float before = 0.f, mu_c = 0.f;
+    float* mine = nullptr;
+    if (mu && slot >= 0 && in) {
+      mine = state + (size_t)slot * width + c;
+      before = first ? 0.f : *mine;
+      mu_c = mu[c];
+    }
+    __syncthreads();
+    float u = 0.f;
+    if (!y) {
+#pragma unroll
+      for (int s = 0; s < SMAX; ++s) if (s < S) u = fmaf(k.read[s], old[s], u);
+    } else {
+#pragma unroll
+      for (int to = 0; to < SMAX; ++to) {
+        if (to < S) {
+          float v = 0.f;
+#pragma unroll
+          for (int s = 0; s < SMAX; ++s) if (s < S) v = fmaf(k.mix[s * MAX_STREAMS + to], old[s], v);
+          v = fmaf(k.out[to], add, v);
+          if (store && in) x[(size_t)to * width + c] = v;
+          u = fmaf(k.read[to], v, u);
+        }
+      }
+    }
+    const float total = block_sum(u * u, scratch);
+    float h = u * (1.0f / sqrtf(total / (float)width + eps) * gain[0]);
+    if (mine) {
+      *mine = h;
+      h = fmaf(before - h, mu_c, h);
+    }
+    if (in) st(out + (size_t)i * width + c, h);
+    return;
+  }
+  __syncthreads();
   float kept[KEPT_COLUMNS], sq = 0.f;
   int n = 0;
   for (int c = threadIdx.x; c < width; c += blockDim.x, ++n) {
-    const float u = stream_column(x, yr, scale, k, S, width, c, store);
+    const float u = stream_column<TY, SMAX>(x, yr, scale, k, S, width, c, store);
     if (n < KEPT_COLUMNS) kept[n] = u;
     sq = fmaf(u, u, sq);
   }
@@ -105,7 +158,7 @@ streams_step_kernel(float* __restrict__ streams, const TY* __restrict__ y, const
   for (int c = threadIdx.x; c < width; c += blockDim.x, ++n) {
     // (Past the kept columns the read is made again: from the streams as they are now if they were stored, which
     // adds the same numbers in the same order, else from the old ones.)
-    const float u = n < KEPT_COLUMNS ? kept[n] : stream_column(x, store ? (const TY*)nullptr : yr, scale, k, S, width, c, false);
+    const float u = n < KEPT_COLUMNS ? kept[n] : stream_column<TY, SMAX>(x, store ? (const TY*)nullptr : yr, scale, k, S, width, c, false);
     float h = u * inv;
     if (mu && slot >= 0) {
       float* mine = state + (size_t)slot * width + c;
@@ -178,12 +231,14 @@ extern "C" int ta_streams_step(void* streams, const void* y, const void* mix, co
   // 256 columns; many rows fill the device with workgroups of 256.
   int threads = 256;
   if (n_rows <= 2 * compute_units()) threads = width >= 1024 ? 1024 : (width + WAVE - 1) / WAVE * WAVE;
-#define GO(TY, TO) streams_step_kernel<TY, TO><<<n_rows, threads, 0, stream>>>((float*)streams, (const TY*)y, (const float*)mix, \
+#define GO(TY, TO) if (n_streams <= 4) GO_S(TY, TO, 4); else if (n_streams <= 8) GO_S(TY, TO, 8); else GO_S(TY, TO, 16)
+#define GO_S(TY, TO, SS) streams_step_kernel<TY, TO, SS><<<n_rows, threads, 0, stream>>>((float*)streams, (const TY*)y, (const float*)mix, \
     (const float*)out_coef, (const float*)scale, (const float*)read, (const float*)gain, eps, (TO*)out, (const int*)rows,   \
     width, n_streams, (const float*)mu, (float*)state, (const int*)entry_of_token, (const int*)state_slots,                 \
     (const int*)positions)
-  if (y_dtype == DT_F32) { if (out_dtype == DT_F32) GO(float, float); else return -1; }
-  else { if (out_dtype == DT_F32) GO(bf16_t, float); else GO(bf16_t, bf16_t); }
+  if (y_dtype == DT_F32) { if (out_dtype == DT_F32) { GO(float, float); } else return -1; }
+  else { if (out_dtype == DT_F32) { GO(bf16_t, float); } else { GO(bf16_t, bf16_t); } }
+#undef GO_S
 #undef GO
   return LAUNCH_STATUS();
 }
