@@ -272,7 +272,7 @@ class PlainOps:
             v_pages.copy_(work_v.to(v_pages.dtype))
         return holder[:, :n_q * head_dim].to(weight.dtype).contiguous()
 
-    def fused_norm_gated(self, residual, norm_weight, eps, weight):
+    def fused_norm_gated(self, residual, norm_weight, eps, weight, act=None):
         if norm_weight is None:
             x = residual
         else:
@@ -281,6 +281,10 @@ class PlainOps:
         gate_up = x.to(self.work) @ weight.to(self.work).t()
         inner = weight.shape[0] // 2
         g, u = gate_up[:, :inner], gate_up[:, inner:]
+        if act is not None:
+            alpha, limit, shift = (float(v) for v in act)
+            g, u = torch.clamp(g, max=limit), torch.clamp(u, min=-limit, max=limit)
+            return (g * torch.sigmoid(alpha * g) * (u + shift)).to(weight.dtype)
         return (g * torch.sigmoid(g) * u).to(weight.dtype)
 
     def linear_add(self, x, weight, bias, residual):

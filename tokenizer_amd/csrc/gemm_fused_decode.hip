@@ -190,6 +190,10 @@ fused_decode_kernel(const bf16_t* w, const void* rows_in, void* result, const fl
   for (int ps = 0; ps < PASSES; ++ps)
 #pragma unroll
     for (int r = 0; r < 4; ++r) pre_a[ps][r] = pre_b[ps][r] = 0.f;
+  // EPI_GATED with another activation than silu: its three numbers (alpha, limit, shift) lie where the rotation's table
+  // would: g' = min(g, limit), u' = clamp(u, -limit, limit), g' sigmoid(alpha g') (u' + shift).
+  float act_alpha = 1.f, act_limit = INFINITY, act_shift = 0.f;
+  if (EPI == EPI_GATED && p.cos_sin) { act_alpha = p.cos_sin[0]; act_limit = p.cos_sin[1]; act_shift = p.cos_sin[2]; }
   if (EPI == EPI_RESIDUAL && wave == 0) HELD(bias);
   if (wave == 0 && col < M) {
     if (EPI == EPI_RESIDUAL) {
@@ -355,7 +359,14 @@ fused_decode_kernel(const bf16_t* w, const void* rows_in, void* result, const fl
         bf16_t* dst = p.out + (size_t)m * p.ldc + n;
 #pragma unroll
         for (int r = 0; r < 4; ++r)
-          if (local + r < R && n + r < n_limit) st(dst + r, v0[r] / (1.0f + __expf(-v0[r])) * v1[r]);
+          if (local + r < R && n + r < n_limit) {
+            if (p.cos_sin) {
+              const float gate = fminf(v0[r], act_limit), up = fminf(fmaxf(v1[r], -act_limit), act_limit);
+              st(dst + r, gate / (1.0f + __expf(-act_alpha * gate)) * (up + act_shift));
+            } else {
+              st(dst + r, v0[r] / (1.0f + __expf(-v0[r])) * v1[r]);
+            }
+          }
       } else {
         const int d = p.d, half = d / 2;
         const int slot = pre_slot;
@@ -553,25 +564,30 @@ extern "C" int ta_fused_qkv_rope(const void* x, int lda, const void* w, const vo
 }
 
 // out [m, n/2] = silu(x Wg^T) * (x Wu^T), x = the normalised residual rows, W = [Wg; Wu] of shape [n, k].
+// act: null for silu, else three floats on the device (alpha, limit, shift): g' = min(g, limit), u' = clamp(u, +-limit),
+// out = g' sigmoid(alpha g') (u' + shift).
 extern "C" int ta_fused_norm_gated(const void* residual, const void* norm_weight, float eps, const void* w,
-                                   void* out, int m, int n, int k, int rows, int waves, hipStream_t stream) {
+                                   void* out, int m, int n, int k, int rows, int waves, const void* act,
+                                   hipStream_t stream) {
   if (m <= 0) return 0;
   if (m > 16 || (k & 7) || (n & 1)) return -1;
   FusedArgs a = {};
   a.residual_in = (const float*)residual; a.norm_weight = (const float*)norm_weight; a.eps = eps;
   a.w = (const bf16_t*)w; a.m = m; a.n = n; a.k = k; a.out = (bf16_t*)out; a.ldc = n / 2;
+  a.cos_sin = (const float*)act;
   a.rows = rows_per_gated_workgroup(n / 2, m, k, rows);
   return launch_rows<EPI_GATED, true>(a, (n / 2 + a.rows - 1) / a.rows, waves, stream);
 }
 
 // The same from rows that are normalised already: x bfloat16 [m, k] with row stride lda.
 extern "C" int ta_fused_gated(const void* x, int lda, const void* w, void* out, int m, int n, int k, int rows,
-                              int waves, hipStream_t stream) {
+                              int waves, const void* act, hipStream_t stream) {
   if (m <= 0) return 0;
   if (m > 16 || (k & 7) || (lda & 7) || (n & 1)) return -1;
   FusedArgs a = {};
   a.a = (const bf16_t*)x; a.lda = lda;
   a.w = (const bf16_t*)w; a.m = m; a.n = n; a.k = k; a.out = (bf16_t*)out; a.ldc = n / 2;
+  a.cos_sin = (const float*)act;
   a.rows = stage_rows(m, k) ? rows_per_gated_workgroup(n / 2, m, k, rows) : rows_per_workgroup(n / 2, rows);
   if (stage_rows(m, k)) return launch_rows<EPI_GATED, true>(a, (n / 2 + a.rows - 1) / a.rows, waves, stream);
   return launch_rows<EPI_GATED, false>(a, (n / 2 + a.rows - 1) / a.rows, waves, stream);

@@ -739,10 +739,12 @@ class Ops:
         return (self.use_fused_decode and dtype == torch.bfloat16 and self.FUSED_ROWS < rows <= self.SKINNY_ROWS
                 and weight_elements <= self.ROPE_STORE_WEIGHT)
 
-    def fused_norm_gated(self, residual, norm_weight, eps, weight) -> torch.Tensor:
+    def fused_norm_gated(self, residual, norm_weight, eps, weight, act: torch.Tensor | None = None) -> torch.Tensor:
         """silu(x @ Wg.T) * (x @ Wu.T) with x = rmsnorm(residual), weight = [Wg; Wu]; bfloat16 [M, I].  With
-        `norm_weight` None, `residual` holds the normalised rows in bfloat16 already."""
-        _dev(norm_weight, weight)
+        `norm_weight` None, `residual` holds the normalised rows in bfloat16 already.  `act`: float32 [3] on the
+        device (alpha, limit, shift) for the capped gated activation in place of silu (see `silu_gate`)."""
+        _dev(norm_weight, weight, act)
+        _need(act is None or (act.dtype == torch.float32 and act.numel() == 3), "act is float32 [3]")
         _need(residual.is_cuda and residual.dim() == 2, "the rows must live on the GPU")
         m, k = residual.shape
         if norm_weight is None:
@@ -754,7 +756,7 @@ class Ops:
         _need(weight.dtype == torch.bfloat16 and weight.shape[1] == k and weight.shape[0] % 2 == 0, "gate/up matrix shape")
         _need(m <= self.FUSED_ROWS and k % 8 == 0, "sizes the fused product does not take")
         out = torch.empty((m, weight.shape[0] // 2), dtype=torch.bfloat16, device=residual.device)
-        tail = (_ptr(weight), _ptr(out), m, weight.shape[0], k, self.fused_rows, self.fused_waves, self._stream())
+        tail = (_ptr(weight), _ptr(out), m, weight.shape[0], k, self.fused_rows, self.fused_waves, _ptr(act), self._stream())
         if norm_weight is None:
             status = self.lib.ta_fused_gated(_ptr(residual), residual.stride(0) if m > 1 else k, *tail)
         else:

@@ -128,9 +128,13 @@ class GQAttention(Mixer):
         ops = self.runtime.ops
         can = getattr(ops, "can_rope_store", None)
         behind = None
-        if (can and can(x.shape[0], self.runtime.dtype, self.w_qkv.numel()) and self.d % 32 == 0
-                and cache.group is not None and self.plain):
+        # (The projection with the store in its epilogue does not care what the attention behind it does with
+        # chunks, slopes or sinks: it needs heads of one size and keys and values of the layer's own.)
+        even = self.own_kv and self.dv == self.d and self.d % 32 == 0 and cache.group is not None
+        if can and can(x.shape[0], self.runtime.dtype, self.w_qkv.numel()) and even:
             behind = self.position.epilogue()
+        elif even and not self.plain and _can_fuse(ops, x, self.runtime.dtype) and x.shape[1] % 8 == 0:
+            behind = self.position.epilogue()       # up to sixteen normalised rows: the fused decode projection
         if behind is not None:
             # A few dozen rows: bias, rotation and the cache write ride in the projection's epilogue.
             qkv = ops.fused_norm_qkv_rope(x, None, 0.0, self.w_qkv, self.b_qkv, ctx.positions, behind.cos_sin,

@@ -28,6 +28,7 @@ class GatedDense(FeedForward):
         if spec.activation == "capped_swish":
             limit = float("inf") if spec.act_limit is None else float(spec.act_limit)
             self.act = (float(spec.act_alpha), limit, float(spec.act_up_shift))
+            self.act_numbers = torch.tensor(self.act, dtype=torch.float32, device=runtime.device)   # for kernels that read them
         gate, up, down = tensors["gate_proj.weight"], tensors["up_proj.weight"], tensors["down_proj.weight"]
         # The bfloat16 products read eight elements of K at a time.  An inner width that is no multiple of
         # eight is filled up with zero rows of gate and up and zero columns of down: act(0) * 0 = 0 meets a
@@ -70,5 +71,11 @@ class GatedDense(FeedForward):
 
     def _run(self, x, pending: bool):
         ops = self.runtime.ops
-        act = ops.linear_silu_gate(x, self.w_gate_up) if self.act is None else ops.linear_silu_gate(x, self.w_gate_up, act=self.act)
+        if self.act is None:
+            act = ops.linear_silu_gate(x, self.w_gate_up)
+        elif _can_fuse(ops, x, self.runtime.dtype) and x.shape[1] % 8 == 0:
+            # Up to sixteen normalised rows: the fused decode product with the capped activation in its epilogue.
+            act = ops.fused_norm_gated(x, None, 0.0, self.w_gate_up, act=self.act_numbers)
+        else:
+            act = ops.linear_silu_gate(x, self.w_gate_up, act=self.act)
         return ops.linear(act, self.w_down, pending=True) if pending else ops.linear(act, self.w_down)
