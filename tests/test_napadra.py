@@ -328,6 +328,59 @@ def test_matrix_memory_alone_in_portions(backend, heads, d, dv):
     assert float((torch.cat(got) - want).abs().max()) <= tol * max(1.0, float(want.abs().max()))
 
 
+def _memory_rows(seed, n, heads, d, dv, cap, eps, dtype, forget_shift=2.0):
+    """Rows of q, k, v, g and gate pre-activations of one sequence as the compute dtype holds them, and what the plain
+    function reads from them."""
+    gen = torch.Generator().manual_seed(seed)
+    sizes = [heads * d, heads * d, heads * dv, heads * dv]
+    qkvg = rounded(torch.cat([torch.randn(n, size, generator=gen, dtype=torch.float64) * 0.8 for size in sizes], dim=1), dtype)
+    gates = torch.randn(n, 2 * heads, generator=gen, dtype=torch.float64) * 3.0
+    gates[:, heads:] += forget_shift
+    gates = gates.float().double()
+    w = {"norm": torch.rand(heads * dv, generator=torch.Generator().manual_seed(heads * dv), dtype=torch.float64) + 0.5, "o": torch.eye(heads * dv, dtype=torch.float64),
+         "i.b": torch.zeros(heads, dtype=torch.float64), "f.b": torch.zeros(heads, dtype=torch.float64)}
+    # The plain function makes its own projections: its input is the identity, its weights are the rows themselves.
+    eye = torch.eye(n, dtype=torch.float64)
+    for name, part in zip("qkvg", torch.split(qkvg, sizes, dim=1)):
+        w[name] = part.t().contiguous()
+    w["i"], w["f"] = gates[:, :heads].t().contiguous(), gates[:, heads:].t().contiguous()
+    want = plain.mlstm(eye, {"heads": heads, "dim": d, "vdim": dv, "gate_cap": cap}, w, eps)
+    return qkvg, gates, w["norm"], want
+
+
+@pytest.mark.parametrize("backend", BACKENDS)
+@pytest.mark.parametrize("heads,d,dv,shift", [(2, 16, 24, 2.0), (1, 72, 8, 4.0), (3, 12, 70, -1.0), (1, 130, 66, 6.0)])
+def test_matrix_memory_in_long_portions_beside_single_tokens(backend, heads, d, dv, shift):
+    """Two sequences whose portions run from one row to hundreds, side by side: long portions take the form in chunks of
+    64 tokens, short ones the token-by-token form, and the state passes between the two from step to step."""
+    ops, device, dtype = ops_for(backend)
+    cap, eps = 7.0, 1e-5
+    steps = [(130, 1), (70, 65), (1, 2), (99, 50), (64, 0), (1, 128), (3, 1)]
+    lengths = [sum(a for a, _ in steps), sum(b for _, b in steps)]
+    seqs = [_memory_rows(11 * heads + d + k, lengths[k], heads, d, dv, cap, eps, dtype, shift) for k in range(2)]
+    state = torch.full((5, heads * d * dv + heads * d + heads + 1), float("nan"), device=device)
+    slots, at, got = (3, 1), [0, 0], [[], []]
+    for sizes in steps:
+        live = [k for k in range(2) if sizes[k]]
+        batch = Batch([(at[k], sizes[k], slots[k]) for k in live], device)
+        rows = torch.cat([seqs[k][0][at[k]:at[k] + sizes[k]] for k in live]).to(dtype).to(device).contiguous()
+        gate_rows = torch.cat([seqs[k][1][at[k]:at[k] + sizes[k]] for k in live]).float().to(device).contiguous()
+        read = torch.empty((rows.shape[0], heads * dv), dtype=torch.float32, device=device)
+        ops.mlstm_scan(rows, gate_rows, state, batch.cu_q, batch.first_position, batch.state_slots, read, heads, d, dv, cap)
+        out = torch.empty((rows.shape[0], heads * dv), dtype=dtype, device=device)
+        ops.head_norm_gate(read, seqs[0][2].float().to(device), rows, 2 * heads * d + heads * dv, eps, heads, dv, out)
+        out = out.double().cpu()
+        row = 0
+        for k in live:
+            got[k].append(out[row:row + sizes[k]])
+            row += sizes[k]
+            at[k] += sizes[k]
+    tol = 3e-2 if dtype == torch.bfloat16 else 2e-4
+    for k in range(2):
+        want = seqs[k][3]
+        assert float((torch.cat(got[k]) - want).abs().max()) <= tol * max(1.0, float(want.abs().max())), k
+
+
 def _paged(ops, device, dtype, q, k, v, page_size, chunk, slopes, sinks, scale, first_page=3, as_prompt=False):
     """Attention of every row of q (positions 0..n-1 of one request) over keys and values laid into pages.
     `as_prompt`: the rows are described as one portion of a prompt (the kernels for portions then take them)."""

@@ -220,6 +220,280 @@ mlstm_memory_kernel(const T* __restrict__ qkvg, int row_stride, const float* __r
   }
 }
 
+// ---------------------------------------------------------------------------------------------------------------
+// The same recurrence in chunks of 64 tokens, for portions of many tokens.  With b_t the sum of the forget gates from
+// the chunk's first token to t, a_t = max over s <= t of (b_t - b_s + i_s) and m_0 the maximum before the chunk, the
+// running maximum is m_t = max(b_t + m_0, a_t), and in terms of the state (C_0, n_0) before the chunk
+//   C_t^T q_t = exp(b_t + m_0 - m_t) C_0^T q_t + sum over s <= t of exp(b_t - b_s + i_s - m_t) (q_t . k_s) v_s,
+// likewise n_t . q_t; no exponent is above 0.  Three kernels: every chunk's own sums as if it started from nothing
+// (all chunks side by side), the states before every chunk (one after the other, an element a thread), the reads (all
+// chunks side by side).  All of it in float; the sums b and the exponents' arguments in double, so that a difference
+// of two long sums keeps its digits.  Products are 64 x 64 tiles through LDS, a 4 x 4 piece a thread.
+#define MC_L 64            // tokens of a chunk, and the side of a tile
+#define MC_LD 65           // floats from one row of a tile in LDS to the next
+
+struct chunk_place { int entry, index, count, lo, n; };     // the entry, which of its `count` chunks, first row, rows
+
+// Chunk g of the batch: entries in their order, each with as many chunks as its rows need.
+__device__ __forceinline__ bool find_chunk(const int* __restrict__ cu_q, int n_entries, int g, chunk_place& p) {
+  int base = 0;
+  for (int e = 0; e < n_entries; ++e) {
+    const int lo = cu_q[e], len = cu_q[e + 1] - lo;
+    const int count = len > 0 ? (len + MC_L - 1) / MC_L : 0;
+    if (g < base + count) {
+      p.entry = e; p.index = g - base; p.count = count; p.lo = lo + p.index * MC_L;
+      p.n = min(MC_L, lo + len - p.lo);
+      return true;
+    }
+    base += count;
+  }
+  return false;
+}
+
+// The chunk's log input gates i_s, sums of forget gates b_s and maxima a_s as above (entries from n on repeat n - 1).
+__device__ __forceinline__ void chunk_gates(const float* __restrict__ gates, int gate_stride, int heads, int h, float cap,
+                                            int lo, int n, float* i_s, double* b_s, float* a_s) {
+  const int tid = threadIdx.x;
+  if (tid < MC_L) {
+    float gi = -INFINITY, gf = 0.f;
+    if (tid < n) {
+      gi = capped(gates[(size_t)(lo + tid) * gate_stride + h], cap);
+      gf = log_sigmoid(capped(gates[(size_t)(lo + tid) * gate_stride + heads + h], cap));
+    }
+    i_s[tid] = gi; a_s[tid] = gf;                            // a_s holds f until the chain below has passed
+  }
+  __syncthreads();
+  if (tid == 0) {
+    double b = 0.0;
+    float a = -INFINITY;
+    for (int s = 0; s < MC_L; ++s) {
+      if (s < n) { const float f = a_s[s]; b += (double)f; a = fmaxf(f + a, i_s[s]); }
+      b_s[s] = b; a_s[s] = a;
+    }
+  }
+  __syncthreads();
+}
+
+// A tile of rows [row0, row0 + n) x columns [col0, col0 + 64) of `src` (rows of `stride` elements) into LDS, zeros
+// outside n rows and `cols` columns; `scale` times every element.
+template <typename T>
+__device__ __forceinline__ void load_tile(float (*tile)[MC_LD], const T* __restrict__ src, size_t stride, int n, int cols,
+                                          float scale) {
+  for (int x = threadIdx.x; x < MC_L * MC_L; x += 4 * WAVE) {
+    const int r = x >> 6, c = x & 63;
+    tile[r][c] = (r < n && c < cols) ? ld(src + (size_t)r * stride + c) * scale : 0.f;
+  }
+}
+
+// Every chunk from nothing: local[g, h] = [sum_s w_s k_s v_s^T (d x dv) | sum_s w_s k_s (d)] with
+// w_s = exp(b_last - b_s + i_s - a_last), and ends[g, h] = (b_last, a_last).
+template <typename T>
+__global__ void __launch_bounds__(4 * WAVE)
+mlstm_chunk_local_kernel(const T* __restrict__ qkvg, int row_stride, const float* __restrict__ gates, int gate_stride,
+                         const int* __restrict__ cu_q, int n_entries, float* __restrict__ local, float* __restrict__ ends,
+                         int heads, int d, int dv, float cap) {
+  __shared__ float k_s[MC_L][MC_LD], v_s[MC_L][MC_LD];
+  __shared__ float i_s[MC_L], a_s[MC_L], w_s[MC_L];
+  __shared__ double b_s[MC_L];
+  const int g = blockIdx.x, h = blockIdx.y, tid = threadIdx.x, ty = tid >> 4, tx = tid & 15;
+  chunk_place p;
+  if (!find_chunk(cu_q, n_entries, g, p)) return;
+  const int n = p.n;
+  chunk_gates(gates, gate_stride, heads, h, cap, p.lo, n, i_s, b_s, a_s);
+  if (tid < MC_L)
+    w_s[tid] = tid < n ? expf((float)((b_s[n - 1] - b_s[tid]) + (double)i_s[tid] - (double)a_s[n - 1])) : 0.f;
+  if (tid == 0) {
+    ends[((size_t)g * heads + h) * 2] = (float)b_s[n - 1];
+    ends[((size_t)g * heads + h) * 2 + 1] = a_s[n - 1];
+  }
+  __syncthreads();
+  const size_t total = (size_t)d * dv + d;
+  float* dst = local + ((size_t)g * heads + h) * total;
+  const T* rows = qkvg + (size_t)p.lo * row_stride;
+  for (int j0 = 0; j0 < d; j0 += MC_L) {
+    for (int x = tid; x < MC_L * MC_L; x += 4 * WAVE) {      // k rows times their weights
+      const int s = x >> 6, jj = x & 63;
+      k_s[s][jj] = (s < n && j0 + jj < d) ? ld(rows + (size_t)s * row_stride + (size_t)(heads + h) * d + j0 + jj) * w_s[s] : 0.f;
+    }
+    __syncthreads();
+    if (tid < MC_L && j0 + tid < d) {
+      float sum = 0.f;
+      for (int s = 0; s < n; ++s) sum += k_s[s][tid];
+      dst[(size_t)d * dv + j0 + tid] = sum;
+    }
+    for (int c0 = 0; c0 < dv; c0 += MC_L) {
+      load_tile(v_s, rows + (size_t)2 * heads * d + (size_t)h * dv + c0, (size_t)row_stride, n, dv - c0, 1.f);
+      __syncthreads();
+      float acc[4][4] = {};
+      for (int s = 0; s < n; ++s) {
+        float kk[4], vv[4];
+#pragma unroll
+        for (int r = 0; r < 4; ++r) { kk[r] = k_s[s][ty * 4 + r]; vv[r] = v_s[s][tx + 16 * r]; }
+#pragma unroll
+        for (int r = 0; r < 4; ++r)
+#pragma unroll
+          for (int c = 0; c < 4; ++c) acc[r][c] = fmaf(kk[r], vv[c], acc[r][c]);
+      }
+#pragma unroll
+      for (int r = 0; r < 4; ++r)
+#pragma unroll
+        for (int c = 0; c < 4; ++c) {
+          const int j = j0 + ty * 4 + r, col = c0 + tx + 16 * c;
+          if (j < d && col < dv) dst[(size_t)j * dv + col] = acc[r][c];
+        }
+      __syncthreads();                                       // the tiles are free again
+    }
+  }
+}
+
+// From chunk to chunk, an element of [C | n] a thread: local[g, h] becomes the state before chunk g, the state after
+// the entry's last chunk goes into its slot, m_start[g, h] is the maximum before chunk g.  (The slot's m is written by
+// the reads' kernel: every workgroup here reads it.)
+__global__ void __launch_bounds__(4 * WAVE)
+mlstm_chunk_carry_kernel(float* __restrict__ state, size_t state_stride, const int* __restrict__ cu_q,
+                         const int* __restrict__ first_position, const int* __restrict__ state_slots,
+                         float* local, const float* __restrict__ ends, float* __restrict__ m_start,
+                         int heads, int d, int dv) {
+  const int e = blockIdx.x, h = blockIdx.y, tid = threadIdx.x;
+  const int len = cu_q[e + 1] - cu_q[e];
+  if (len <= 0) return;
+  int base = 0;
+  for (int x = 0; x < e; ++x) {
+    const int l = cu_q[x + 1] - cu_q[x];
+    base += l > 0 ? (l + MC_L - 1) / MC_L : 0;
+  }
+  const int count = (len + MC_L - 1) / MC_L;
+  const size_t plane = (size_t)d * dv, total = plane + d, idx = (size_t)blockIdx.z * (4 * WAVE) + tid;
+  const bool live = idx < total;
+  float* row = state + (size_t)state_slots[e] * state_stride;
+  float* mine = idx < plane ? row + (size_t)h * plane + idx : row + (size_t)heads * plane + (size_t)h * d + (idx - plane);
+  const bool fresh = first_position[e] == 0;
+  float x = (live && !fresh) ? *mine : 0.f;
+  float m = fresh ? 0.f : row[(size_t)heads * plane + (size_t)heads * d + h];
+  const size_t step = (size_t)heads * total;
+  float* src = local + ((size_t)base * heads + h) * total + idx;
+  float next = live ? src[0] : 0.f;
+  for (int c = 0; c < count; ++c) {
+    const float now = next;
+    if (live) {
+      src[(size_t)c * step] = x;
+      if (c + 1 < count) next = src[(size_t)(c + 1) * step];
+    }
+    const float b_last = ends[((size_t)(base + c) * heads + h) * 2], a_last = ends[((size_t)(base + c) * heads + h) * 2 + 1];
+    const float m_new = fmaxf(b_last + m, a_last);
+    if (blockIdx.z == 0 && tid == 0) m_start[(size_t)(base + c) * heads + h] = m;
+    x = fmaf(expf(b_last + m - m_new), x, expf(a_last - m_new) * now);
+    m = m_new;
+  }
+  if (live) *mine = x;
+}
+
+// The reads of a chunk's tokens from the state before the chunk (`start`, what the carry left in `local`) and the
+// chunk's own keys and values.
+template <typename T>
+__global__ void __launch_bounds__(4 * WAVE)
+mlstm_chunk_read_kernel(const T* __restrict__ qkvg, int row_stride, const float* __restrict__ gates, int gate_stride,
+                        float* __restrict__ state, size_t state_stride, const int* __restrict__ cu_q,
+                        const int* __restrict__ state_slots, int n_entries, const float* __restrict__ local,
+                        const float* __restrict__ m_start, float* __restrict__ out, int heads, int d, int dv, float cap) {
+  __shared__ float q_s[MC_L][MC_LD], k_s[MC_L][MC_LD], p_s[MC_L][MC_LD];
+  __shared__ float i_s[MC_L], a_s[MC_L], m_s[MC_L], w0_s[MC_L], div_s[MC_L];
+  __shared__ double b_s[MC_L];
+  const int g = blockIdx.x, h = blockIdx.y, tid = threadIdx.x, ty = tid >> 4, tx = tid & 15;
+  chunk_place p;
+  if (!find_chunk(cu_q, n_entries, g, p)) return;
+  const int n = p.n;
+  chunk_gates(gates, gate_stride, heads, h, cap, p.lo, n, i_s, b_s, a_s);
+  const float m0 = m_start[(size_t)g * heads + h];
+  if (tid < MC_L) {
+    const float m = fmaxf((float)(b_s[tid] + (double)m0), a_s[tid]);
+    m_s[tid] = m;
+    w0_s[tid] = expf((float)(b_s[tid] + (double)m0 - (double)m));
+    if (tid == n - 1 && p.index == p.count - 1)
+      state[(size_t)state_slots[p.entry] * state_stride + (size_t)heads * d * dv + (size_t)heads * d + h] = m;
+  }
+  const size_t plane = (size_t)d * dv;
+  const float* start = local + ((size_t)g * heads + h) * (plane + d);
+  const T* rows = qkvg + (size_t)p.lo * row_stride;
+  const float q_scale = 1.0f / sqrtf((float)d);
+  // q_t . k_s over the whole of d, and n_0 . q_t (thread t).
+  float acc[4][4] = {};
+  float dn = 0.f;
+  for (int j0 = 0; j0 < d; j0 += MC_L) {
+    const int lim = min(MC_L, d - j0);
+    __syncthreads();
+    load_tile(q_s, rows + (size_t)h * d + j0, (size_t)row_stride, n, lim, q_scale);
+    load_tile(k_s, rows + (size_t)(heads + h) * d + j0, (size_t)row_stride, n, lim, 1.f);
+    __syncthreads();
+    for (int jj = 0; jj < lim; ++jj) {
+      float qq[4], kk[4];
+#pragma unroll
+      for (int r = 0; r < 4; ++r) { qq[r] = q_s[ty * 4 + r][jj]; kk[r] = k_s[tx + 16 * r][jj]; }
+#pragma unroll
+      for (int r = 0; r < 4; ++r)
+#pragma unroll
+        for (int c = 0; c < 4; ++c) acc[r][c] = fmaf(qq[r], kk[c], acc[r][c]);
+    }
+    if (tid < MC_L)
+      for (int jj = 0; jj < lim; ++jj) dn = fmaf(q_s[tid][jj], start[plane + j0 + jj], dn);
+  }
+  // Scores times their decays; nothing above the diagonal or past the chunk's rows.
+#pragma unroll
+  for (int r = 0; r < 4; ++r)
+#pragma unroll
+    for (int c = 0; c < 4; ++c) {
+      const int t = ty * 4 + r, s = tx + 16 * c;
+      float w = 0.f;
+      if (s <= t && t < n) w = acc[r][c] * expf((float)((b_s[t] - b_s[s]) + (double)i_s[s] - (double)m_s[t]));
+      p_s[t][s] = w;
+    }
+  __syncthreads();
+  if (tid < MC_L) {
+    float dot = w0_s[tid] * dn;
+    for (int s = 0; s <= tid; ++s) dot += p_s[tid][s];
+    div_s[tid] = fmaxf(fabsf(dot), expf(-m_s[tid])) + 1e-6f;
+  }
+  for (int c0 = 0; c0 < dv; c0 += MC_L) {
+    float own[4][4] = {}, old[4][4] = {};
+    __syncthreads();                                         // k_s is free, div_s is written
+    load_tile(k_s, rows + (size_t)2 * heads * d + (size_t)h * dv + c0, (size_t)row_stride, n, dv - c0, 1.f);
+    __syncthreads();
+    for (int s = 0; s < n; ++s) {
+      float pp[4], vv[4];
+#pragma unroll
+      for (int r = 0; r < 4; ++r) { pp[r] = p_s[ty * 4 + r][s]; vv[r] = k_s[s][tx + 16 * r]; }
+#pragma unroll
+      for (int r = 0; r < 4; ++r)
+#pragma unroll
+        for (int c = 0; c < 4; ++c) own[r][c] = fmaf(pp[r], vv[c], own[r][c]);
+    }
+    for (int j0 = 0; j0 < d; j0 += MC_L) {
+      const int lim = min(MC_L, d - j0);
+      __syncthreads();
+      load_tile(q_s, rows + (size_t)h * d + j0, (size_t)row_stride, n, lim, q_scale);
+      load_tile(k_s, start + (size_t)j0 * dv + c0, (size_t)dv, lim, dv - c0, 1.f);
+      __syncthreads();
+      for (int jj = 0; jj < lim; ++jj) {
+        float qq[4], cc[4];
+#pragma unroll
+        for (int r = 0; r < 4; ++r) { qq[r] = q_s[ty * 4 + r][jj]; cc[r] = k_s[jj][tx + 16 * r]; }
+#pragma unroll
+        for (int r = 0; r < 4; ++r)
+#pragma unroll
+          for (int c = 0; c < 4; ++c) old[r][c] = fmaf(qq[r], cc[c], old[r][c]);
+      }
+    }
+#pragma unroll
+    for (int r = 0; r < 4; ++r)
+#pragma unroll
+      for (int c = 0; c < 4; ++c) {
+        const int t = ty * 4 + r, col = c0 + tx + 16 * c;
+        if (t < n && col < dv)
+          out[(size_t)(p.lo + t) * heads * dv + (size_t)h * dv + col] = fmaf(w0_s[t], old[r][c], own[r][c]) / div_s[t];
+      }
+  }
+}
+
 // out[t, h, :] = read[t, h, :] / sqrt(mean(read[t, h, :]^2) + eps) * weight[h, :] * sigmoid(gate[t, h, :]); `gate` lies
 // in rows of `gate_stride` elements, from column `gate_offset` on.  One wave per (token, head).
 template <typename T>
@@ -262,6 +536,32 @@ extern "C" int ta_mlstm_scan(const void* qkvg, int row_stride, const void* gates
 #undef BOTH
 #undef PASS2
 #undef PASS1
+  return LAUNCH_STATUS();
+}
+
+// The chunked form of ta_mlstm_scan.  scratch: float [max_chunks * heads * (d dv + d + 3)], with max_chunks at least the
+// number of 64-token chunks of all entries together (rows / 64 + entries is enough).
+extern "C" int ta_mlstm_chunked(const void* qkvg, int row_stride, const void* gates, int gate_stride, void* state,
+                                long state_stride, const void* cu_q, const void* first_position, const void* state_slots,
+                                void* scratch, void* out, int n_entries, int max_chunks, int heads, int d, int dv, float cap,
+                                int dtype, hipStream_t stream) {
+  if (n_entries <= 0 || max_chunks <= 0) return 0;
+  if (d < 1 || dv < 1 || heads < 1 || state_stride < (long)heads * d * dv + (long)heads * d + heads) return -1;
+  const size_t total = (size_t)d * dv + d;
+  float* local = (float*)scratch;
+  float* ends = local + (size_t)max_chunks * heads * total;
+  float* m_start = ends + (size_t)max_chunks * heads * 2;
+  dim3 per_chunk(max_chunks, heads), per_entry(n_entries, heads, (unsigned)((total + 4 * WAVE - 1) / (4 * WAVE)));
+#define CHUNKED(TT)                                                                                                        \
+  mlstm_chunk_local_kernel<TT><<<per_chunk, 4 * WAVE, 0, stream>>>((const TT*)qkvg, row_stride, (const float*)gates,        \
+      gate_stride, (const int*)cu_q, n_entries, local, ends, heads, d, dv, cap);                                           \
+  mlstm_chunk_carry_kernel<<<per_entry, 4 * WAVE, 0, stream>>>((float*)state, (size_t)state_stride, (const int*)cu_q,       \
+      (const int*)first_position, (const int*)state_slots, local, ends, m_start, heads, d, dv);                            \
+  mlstm_chunk_read_kernel<TT><<<per_chunk, 4 * WAVE, 0, stream>>>((const TT*)qkvg, row_stride, (const float*)gates,         \
+      gate_stride, (float*)state, (size_t)state_stride, (const int*)cu_q, (const int*)state_slots, n_entries, local,       \
+      m_start, (float*)out, heads, d, dv, cap)
+  if (dtype == DT_F32) { CHUNKED(float); } else { CHUNKED(bf16_t); }
+#undef CHUNKED
   return LAUNCH_STATUS();
 }
 

@@ -153,7 +153,7 @@ class Ops:
                      "ta_fused_norm_gated", "ta_fused_linear_residual", "ta_fused_qkv_rope", "ta_fused_gated",
                      "ta_splitk_reduce", "ta_splitk_add_rmsnorm", "ta_argmax", "ta_argmax_next_step", "ta_sample",
                      "ta_sample_workspace_words", "ta_library_gemm_bf16", "ta_compute_units", "ta_read_stream",
-                     "ta_embedding_streams", "ta_streams_step", "ta_token_shift", "ta_mlstm_scan", "ta_head_norm_gate",
+                     "ta_embedding_streams", "ta_streams_step", "ta_token_shift", "ta_mlstm_scan", "ta_mlstm_chunked", "ta_head_norm_gate",
                      "ta_capped_gate"):
             getattr(self.lib, name).restype = ctypes.c_int
         self.lib.ta_library_gemm_bf16.argtypes = [ctypes.c_void_p] * 4 + [ctypes.c_int] * 5 + [
@@ -862,6 +862,8 @@ class Ops:
         return out
 
     # -------------------------------------------------------------- matrix memory
+    MLSTM_CHUNKED_FROM = 48      # rows beyond one per entry from which the recurrence runs in chunks
+
     def mlstm_scan(self, qkvg: torch.Tensor, gates: torch.Tensor, state: torch.Tensor, cu_q: torch.Tensor,
                    first_position: torch.Tensor, state_slots: torch.Tensor, out: torch.Tensor,
                    heads: int, d: int, dv: int, cap: float) -> torch.Tensor:
@@ -879,6 +881,15 @@ class Ops:
         _need(out.dtype == torch.float32 and tuple(out.shape) == (n_tokens, heads * dv), "out float32 [T, heads dv]")
         n_entries = cu_q.numel() - 1
         _need(first_position.numel() == n_entries == state_slots.numel(), "one first position and slot per entry")
+        if n_tokens - n_entries >= self.MLSTM_CHUNKED_FROM:
+            # Portions of many rows: chunks of 64 tokens side by side, the state carried from chunk to chunk.
+            max_chunks = n_tokens // 64 + n_entries
+            scratch = torch.empty(max_chunks * heads * (d * dv + d + 3), dtype=torch.float32, device=qkvg.device)
+            self._check(self.lib.ta_mlstm_chunked(_ptr(qkvg), qkvg.shape[1], _ptr(gates), gates.shape[1], _ptr(state),
+                                                  ctypes.c_long(state.shape[1]), _ptr(cu_q), _ptr(first_position),
+                                                  _ptr(state_slots), _ptr(scratch), _ptr(out), n_entries, max_chunks, heads, d,
+                                                  dv, ctypes.c_float(cap), _code(qkvg.dtype), self._stream()), "mlstm_chunked")
+            return out
         coef = torch.empty((n_tokens, heads, 3), dtype=torch.float32, device=qkvg.device)
         self._check(self.lib.ta_mlstm_scan(_ptr(qkvg), qkvg.shape[1], _ptr(gates), gates.shape[1], _ptr(state),
                                            ctypes.c_long(state.shape[1]), _ptr(cu_q), _ptr(first_position), _ptr(state_slots),
