@@ -250,7 +250,8 @@ __device__ __forceinline__ bool find_chunk(const int* __restrict__ cu_q, int n_e
   return false;
 }
 
-// The chunk's log input gates i_s, sums of forget gates b_s and maxima a_s as above (entries from n on repeat n - 1).
+// The chunk's log input gates i_s, sums of forget gates b_s and maxima a_s as above (entries from n on repeat n - 1),
+// by the first wave: sums and maxima along the lanes in six steps each, a_t = b_t + max over s <= t of (i_s - b_s).
 __device__ __forceinline__ void chunk_gates(const float* __restrict__ gates, int gate_stride, int heads, int h, float cap,
                                             int lo, int n, float* i_s, double* b_s, float* a_s) {
   const int tid = threadIdx.x;
@@ -260,16 +261,19 @@ __device__ __forceinline__ void chunk_gates(const float* __restrict__ gates, int
       gi = capped(gates[(size_t)(lo + tid) * gate_stride + h], cap);
       gf = log_sigmoid(capped(gates[(size_t)(lo + tid) * gate_stride + heads + h], cap));
     }
-    i_s[tid] = gi; a_s[tid] = gf;                            // a_s holds f until the chain below has passed
-  }
-  __syncthreads();
-  if (tid == 0) {
-    double b = 0.0;
-    float a = -INFINITY;
-    for (int s = 0; s < MC_L; ++s) {
-      if (s < n) { const float f = a_s[s]; b += (double)f; a = fmaxf(f + a, i_s[s]); }
-      b_s[s] = b; a_s[s] = a;
+    double b = (double)gf;
+#pragma unroll
+    for (int off = 1; off < MC_L; off <<= 1) {
+      const double other = __shfl_up(b, off);
+      if (tid >= off) b += other;
     }
+    double z = (double)gi - b;
+#pragma unroll
+    for (int off = 1; off < MC_L; off <<= 1) {
+      const double other = __shfl_up(z, off);
+      if (tid >= off) z = fmax(z, other);
+    }
+    i_s[tid] = gi; b_s[tid] = b; a_s[tid] = (float)(b + z);
   }
   __syncthreads();
 }
@@ -279,10 +283,16 @@ __device__ __forceinline__ void chunk_gates(const float* __restrict__ gates, int
 template <typename T>
 __device__ __forceinline__ void load_tile(float (*tile)[MC_LD], const T* __restrict__ src, size_t stride, int n, int cols,
                                           float scale) {
-  for (int x = threadIdx.x; x < MC_L * MC_L; x += 4 * WAVE) {
-    const int r = x >> 6, c = x & 63;
-    tile[r][c] = (r < n && c < cols) ? ld(src + (size_t)r * stride + c) * scale : 0.f;
+  constexpr int EACH = MC_L * MC_L / (4 * WAVE);             // all of a thread's elements are asked for before any is used
+  const int c = threadIdx.x & 63, r0 = threadIdx.x >> 6;
+  float got[EACH];
+#pragma unroll
+  for (int x = 0; x < EACH; ++x) {
+    const int r = r0 + 4 * x;
+    got[x] = (r < n && c < cols) ? ld(src + (size_t)r * stride + c) : 0.f;
   }
+#pragma unroll
+  for (int x = 0; x < EACH; ++x) tile[r0 + 4 * x][c] = got[x] * scale;
 }
 
 // Every chunk from nothing: local[g, h] = [sum_s w_s k_s v_s^T (d x dv) | sum_s w_s k_s (d)] with
@@ -311,21 +321,21 @@ mlstm_chunk_local_kernel(const T* __restrict__ qkvg, int row_stride, const float
   float* dst = local + ((size_t)g * heads + h) * total;
   const T* rows = qkvg + (size_t)p.lo * row_stride;
   for (int j0 = 0; j0 < d; j0 += MC_L) {
-    for (int x = tid; x < MC_L * MC_L; x += 4 * WAVE) {      // k rows times their weights
-      const int s = x >> 6, jj = x & 63;
-      k_s[s][jj] = (s < n && j0 + jj < d) ? ld(rows + (size_t)s * row_stride + (size_t)(heads + h) * d + j0 + jj) * w_s[s] : 0.f;
-    }
+    load_tile(k_s, rows + (size_t)(heads + h) * d + j0, (size_t)row_stride, n, d - j0, 1.f);
+    for (int x = 0; x < MC_L * MC_L / (4 * WAVE); ++x) k_s[(tid >> 6) + 4 * x][tid & 63] *= w_s[(tid >> 6) + 4 * x];   // a thread's own
     __syncthreads();
     if (tid < MC_L && j0 + tid < d) {
       float sum = 0.f;
-      for (int s = 0; s < n; ++s) sum += k_s[s][tid];
+#pragma unroll 16
+      for (int s = 0; s < MC_L; ++s) sum += k_s[s][tid];       // rows from n on hold zeros
       dst[(size_t)d * dv + j0 + tid] = sum;
     }
     for (int c0 = 0; c0 < dv; c0 += MC_L) {
       load_tile(v_s, rows + (size_t)2 * heads * d + (size_t)h * dv + c0, (size_t)row_stride, n, dv - c0, 1.f);
       __syncthreads();
       float acc[4][4] = {};
-      for (int s = 0; s < n; ++s) {
+#pragma unroll 8
+      for (int s = 0; s < MC_L; ++s) {
         float kk[4], vv[4];
 #pragma unroll
         for (int r = 0; r < 4; ++r) { kk[r] = k_s[s][ty * 4 + r]; vv[r] = v_s[s][tx + 16 * r]; }
@@ -395,9 +405,9 @@ __global__ void __launch_bounds__(4 * WAVE)
 mlstm_chunk_read_kernel(const T* __restrict__ qkvg, int row_stride, const float* __restrict__ gates, int gate_stride,
                         float* __restrict__ state, size_t state_stride, const int* __restrict__ cu_q,
                         const int* __restrict__ state_slots, int n_entries, const float* __restrict__ local,
-                        const float* __restrict__ m_start, float* __restrict__ out, int heads, int d, int dv, float cap) {
+                        const float* __restrict__ ends, const float* __restrict__ m_start, float* __restrict__ out, int heads, int d, int dv, float cap) {
   __shared__ float q_s[MC_L][MC_LD], k_s[MC_L][MC_LD], p_s[MC_L][MC_LD];
-  __shared__ float i_s[MC_L], a_s[MC_L], m_s[MC_L], w0_s[MC_L], div_s[MC_L];
+  __shared__ float i_s[MC_L], a_s[MC_L], m_s[MC_L], w0_s[MC_L], div_s[MC_L], n0_s[MC_L];
   __shared__ double b_s[MC_L];
   const int g = blockIdx.x, h = blockIdx.y, tid = threadIdx.x, ty = tid >> 4, tx = tid & 15;
   chunk_place p;
@@ -405,12 +415,14 @@ mlstm_chunk_read_kernel(const T* __restrict__ qkvg, int row_stride, const float*
   const int n = p.n;
   chunk_gates(gates, gate_stride, heads, h, cap, p.lo, n, i_s, b_s, a_s);
   const float m0 = m_start[(size_t)g * heads + h];
+  // After the entry's last chunk the slot's maximum is the one the carried state was scaled to, by the same operations.
+  if (tid == 0 && p.index == p.count - 1)
+    state[(size_t)state_slots[p.entry] * state_stride + (size_t)heads * d * dv + (size_t)heads * d + h] =
+        fmaxf(ends[((size_t)g * heads + h) * 2] + m0, ends[((size_t)g * heads + h) * 2 + 1]);
   if (tid < MC_L) {
     const float m = fmaxf((float)(b_s[tid] + (double)m0), a_s[tid]);
     m_s[tid] = m;
     w0_s[tid] = expf((float)(b_s[tid] + (double)m0 - (double)m));
-    if (tid == n - 1 && p.index == p.count - 1)
-      state[(size_t)state_slots[p.entry] * state_stride + (size_t)heads * d * dv + (size_t)heads * d + h] = m;
   }
   const size_t plane = (size_t)d * dv;
   const float* start = local + ((size_t)g * heads + h) * (plane + d);
@@ -424,8 +436,10 @@ mlstm_chunk_read_kernel(const T* __restrict__ qkvg, int row_stride, const float*
     __syncthreads();
     load_tile(q_s, rows + (size_t)h * d + j0, (size_t)row_stride, n, lim, q_scale);
     load_tile(k_s, rows + (size_t)(heads + h) * d + j0, (size_t)row_stride, n, lim, 1.f);
+    if (tid < MC_L) n0_s[tid] = tid < lim ? start[plane + j0 + tid] : 0.f;
     __syncthreads();
-    for (int jj = 0; jj < lim; ++jj) {
+#pragma unroll 8
+    for (int jj = 0; jj < MC_L; ++jj) {                      // columns from lim on hold zeros
       float qq[4], kk[4];
 #pragma unroll
       for (int r = 0; r < 4; ++r) { qq[r] = q_s[ty * 4 + r][jj]; kk[r] = k_s[tx + 16 * r][jj]; }
@@ -434,8 +448,10 @@ mlstm_chunk_read_kernel(const T* __restrict__ qkvg, int row_stride, const float*
 #pragma unroll
         for (int c = 0; c < 4; ++c) acc[r][c] = fmaf(qq[r], kk[c], acc[r][c]);
     }
-    if (tid < MC_L)
-      for (int jj = 0; jj < lim; ++jj) dn = fmaf(q_s[tid][jj], start[plane + j0 + jj], dn);
+    if (tid < MC_L) {
+#pragma unroll 16
+      for (int jj = 0; jj < MC_L; ++jj) dn = fmaf(q_s[tid][jj], n0_s[jj], dn);
+    }
   }
   // Scores times their decays; nothing above the diagonal or past the chunk's rows.
 #pragma unroll
@@ -450,7 +466,8 @@ mlstm_chunk_read_kernel(const T* __restrict__ qkvg, int row_stride, const float*
   __syncthreads();
   if (tid < MC_L) {
     float dot = w0_s[tid] * dn;
-    for (int s = 0; s <= tid; ++s) dot += p_s[tid][s];
+#pragma unroll 16
+    for (int s = 0; s < MC_L; ++s) dot += p_s[tid][s];       // zeros above the diagonal
     div_s[tid] = fmaxf(fabsf(dot), expf(-m_s[tid])) + 1e-6f;
   }
   for (int c0 = 0; c0 < dv; c0 += MC_L) {
@@ -458,7 +475,8 @@ mlstm_chunk_read_kernel(const T* __restrict__ qkvg, int row_stride, const float*
     __syncthreads();                                         // k_s is free, div_s is written
     load_tile(k_s, rows + (size_t)2 * heads * d + (size_t)h * dv + c0, (size_t)row_stride, n, dv - c0, 1.f);
     __syncthreads();
-    for (int s = 0; s < n; ++s) {
+#pragma unroll 8
+    for (int s = 0; s < MC_L; ++s) {
       float pp[4], vv[4];
 #pragma unroll
       for (int r = 0; r < 4; ++r) { pp[r] = p_s[ty * 4 + r][s]; vv[r] = k_s[s][tx + 16 * r]; }
@@ -473,7 +491,8 @@ mlstm_chunk_read_kernel(const T* __restrict__ qkvg, int row_stride, const float*
       load_tile(q_s, rows + (size_t)h * d + j0, (size_t)row_stride, n, lim, q_scale);
       load_tile(k_s, start + (size_t)j0 * dv + c0, (size_t)dv, lim, dv - c0, 1.f);
       __syncthreads();
-      for (int jj = 0; jj < lim; ++jj) {
+#pragma unroll 8
+      for (int jj = 0; jj < MC_L; ++jj) {
         float qq[4], cc[4];
 #pragma unroll
         for (int r = 0; r < 4; ++r) { qq[r] = q_s[ty * 4 + r][jj]; cc[r] = k_s[jj][tx + 16 * r]; }
@@ -559,7 +578,7 @@ extern "C" int ta_mlstm_chunked(const void* qkvg, int row_stride, const void* ga
       (const int*)first_position, (const int*)state_slots, local, ends, m_start, heads, d, dv);                            \
   mlstm_chunk_read_kernel<TT><<<per_chunk, 4 * WAVE, 0, stream>>>((const TT*)qkvg, row_stride, (const float*)gates,         \
       gate_stride, (float*)state, (size_t)state_stride, (const int*)cu_q, (const int*)state_slots, n_entries, local,       \
-      m_start, (float*)out, heads, d, dv, cap)
+      ends, m_start, (float*)out, heads, d, dv, cap)
   if (dtype == DT_F32) { CHUNKED(float); } else { CHUNKED(bf16_t); }
 #undef CHUNKED
   return LAUNCH_STATUS();
