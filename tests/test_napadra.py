@@ -473,12 +473,14 @@ def test_the_sink_takes_its_share_and_the_bias_grows_with_distance(backend):
 def test_capped_gated_activation_and_position_vector_alone(backend):
     ops, device, dtype = ops_for(backend)
     gen = torch.Generator().manual_seed(9)
-    x = rounded(torch.randn(7, 2 * 44, generator=gen, dtype=torch.float64) * 2, dtype)
-    out = torch.empty((7, 44), dtype=dtype, device=device)
-    ops.silu_gate(x.to(dtype).to(device), out, act=(1.702, 0.9, 1.0))
-    eye = torch.eye(88, dtype=torch.float64)
-    want = plain.feed_forward(x, {"limit": 0.9}, {"gate": eye[:44], "up": eye[44:], "down": torch.eye(44, dtype=torch.float64)})
-    assert float((out.double().cpu() - want).abs().max()) <= (2e-2 if dtype == torch.bfloat16 else 1e-6) * 2
+    for inner in (44, 72):            # rows of 72 are whole runs of sixteen bytes: the kernel that reads them so
+        x = rounded(torch.randn(7, 2 * inner, generator=gen, dtype=torch.float64) * 2, dtype)
+        out = torch.empty((7, inner), dtype=dtype, device=device)
+        ops.silu_gate(x.to(dtype).to(device), out, act=(1.702, 0.9, 1.0))
+        eye = torch.eye(2 * inner, dtype=torch.float64)
+        want = plain.feed_forward(x, {"limit": 0.9}, {"gate": eye[:inner], "up": eye[inner:],
+                                                       "down": torch.eye(inner, dtype=torch.float64)})
+        assert float((out.double().cpu() - want).abs().max()) <= (2e-2 if dtype == torch.bfloat16 else 1e-6) * 2
     # The embedding with its position vector, into every stream.
     width, vocab = 36, 50
     table = rounded(torch.randn(vocab, width, generator=gen, dtype=torch.float64), dtype)

@@ -227,7 +227,7 @@ mlstm_memory_kernel(const T* __restrict__ qkvg, int row_stride, const float* __r
 //   C_t^T q_t = exp(b_t + m_0 - m_t) C_0^T q_t + sum over s <= t of exp(b_t - b_s + i_s - m_t) (q_t . k_s) v_s,
 // likewise n_t . q_t; no exponent is above 0.  Three kernels: every chunk's own sums as if it started from nothing
 // (all chunks side by side), the states before every chunk (one after the other, an element a thread), the reads (all
-// chunks side by side).  All of it in float; the sums b and the exponents' arguments in double, so that a difference
+// chunks side by side; a workgroup per 64 columns of the values).  All of it in float; the sums b and the exponents' arguments in double, so that a difference
 // of two long sums keeps its digits.  Products are 64 x 64 tiles through LDS, a 4 x 4 piece a thread.
 #define MC_L 64            // tokens of a chunk, and the side of a tile
 #define MC_LD 65           // floats from one row of a tile in LDS to the next
@@ -324,13 +324,14 @@ mlstm_chunk_local_kernel(const T* __restrict__ qkvg, int row_stride, const float
     load_tile(k_s, rows + (size_t)(heads + h) * d + j0, (size_t)row_stride, n, d - j0, 1.f);
     for (int x = 0; x < MC_L * MC_L / (4 * WAVE); ++x) k_s[(tid >> 6) + 4 * x][tid & 63] *= w_s[(tid >> 6) + 4 * x];   // a thread's own
     __syncthreads();
-    if (tid < MC_L && j0 + tid < d) {
+    if (blockIdx.z == 0 && tid < MC_L && j0 + tid < d) {
       float sum = 0.f;
 #pragma unroll 16
       for (int s = 0; s < MC_L; ++s) sum += k_s[s][tid];       // rows from n on hold zeros
       dst[(size_t)d * dv + j0 + tid] = sum;
     }
-    for (int c0 = 0; c0 < dv; c0 += MC_L) {
+    {
+      const int c0 = blockIdx.z * MC_L;                      // this workgroup's 64 columns of v
       load_tile(v_s, rows + (size_t)2 * heads * d + (size_t)h * dv + c0, (size_t)row_stride, n, dv - c0, 1.f);
       __syncthreads();
       float acc[4][4] = {};
@@ -470,7 +471,8 @@ mlstm_chunk_read_kernel(const T* __restrict__ qkvg, int row_stride, const float*
     for (int s = 0; s < MC_L; ++s) dot += p_s[tid][s];       // zeros above the diagonal
     div_s[tid] = fmaxf(fabsf(dot), expf(-m_s[tid])) + 1e-6f;
   }
-  for (int c0 = 0; c0 < dv; c0 += MC_L) {
+  {
+    const int c0 = blockIdx.z * MC_L;                        // this workgroup's 64 columns of the values
     float own[4][4] = {}, old[4][4] = {};
     __syncthreads();                                         // k_s is free, div_s is written
     load_tile(k_s, rows + (size_t)2 * heads * d + (size_t)h * dv + c0, (size_t)row_stride, n, dv - c0, 1.f);
@@ -570,7 +572,7 @@ extern "C" int ta_mlstm_chunked(const void* qkvg, int row_stride, const void* ga
   float* local = (float*)scratch;
   float* ends = local + (size_t)max_chunks * heads * total;
   float* m_start = ends + (size_t)max_chunks * heads * 2;
-  dim3 per_chunk(max_chunks, heads), per_entry(n_entries, heads, (unsigned)((total + 4 * WAVE - 1) / (4 * WAVE)));
+  dim3 per_chunk(max_chunks, heads, (dv + MC_L - 1) / MC_L), per_entry(n_entries, heads, (unsigned)((total + 4 * WAVE - 1) / (4 * WAVE)));
 #define CHUNKED(TT)                                                                                                        \
   mlstm_chunk_local_kernel<TT><<<per_chunk, 4 * WAVE, 0, stream>>>((const TT*)qkvg, row_stride, (const float*)gates,        \
       gate_stride, (const int*)cu_q, n_entries, local, ends, heads, d, dv, cap);                                           \
