@@ -349,7 +349,8 @@ def _memory_rows(seed, n, heads, d, dv, cap, eps, dtype, forget_shift=2.0):
 
 
 @pytest.mark.parametrize("backend", BACKENDS)
-@pytest.mark.parametrize("heads,d,dv,shift", [(2, 16, 24, 2.0), (1, 72, 8, 4.0), (3, 12, 70, -1.0), (1, 130, 66, 6.0)])
+@pytest.mark.parametrize("heads,d,dv,shift", [(2, 16, 24, 2.0), (1, 72, 8, 4.0), (3, 12, 70, -1.0), (1, 130, 66, 6.0),
+                                                (1, 300, 20, 3.0)])
 def test_matrix_memory_in_long_portions_beside_single_tokens(backend, heads, d, dv, shift):
     """Two sequences whose portions run from one row to hundreds, side by side: long portions take the form in chunks of
     64 tokens, short ones the token-by-token form, and the state passes between the two from step to step."""

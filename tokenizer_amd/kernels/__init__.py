@@ -874,15 +874,16 @@ class Ops:
         heads d + heads] (C, n, m; an entry whose first position is 0 starts from zeros); out float32 [T, heads dv]."""
         _dev(qkvg, gates, state, cu_q, first_position, state_slots, out)
         n_tokens = qkvg.shape[0]
-        _need(qkvg.shape[1] >= 2 * heads * d + heads * dv and 0 < d <= 256, "q, k, v do not fit the rows (d up to 256)")
+        _need(qkvg.shape[1] >= 2 * heads * d + heads * dv and d > 0 and dv > 0, "q, k, v do not fit the rows")
         _need(gates.dtype == torch.float32 and gates.shape[0] == n_tokens and gates.shape[1] >= 2 * heads, "gates float32 [T, 2 heads]")
         _need(state.dtype == torch.float32 and state.dim() == 2 and state.shape[1] >= heads * d * dv + heads * d + heads,
               "state rows are too short")
         _need(out.dtype == torch.float32 and tuple(out.shape) == (n_tokens, heads * dv), "out float32 [T, heads dv]")
         n_entries = cu_q.numel() - 1
         _need(first_position.numel() == n_entries == state_slots.numel(), "one first position and slot per entry")
-        if n_tokens - n_entries >= self.MLSTM_CHUNKED_FROM:
-            # Portions of many rows: chunks of 64 tokens side by side, the state carried from chunk to chunk.
+        if n_tokens - n_entries >= self.MLSTM_CHUNKED_FROM or d > 256:
+            # Portions of many rows: chunks of 64 tokens side by side, the state carried from chunk to chunk.  (Heads wider
+            # than the 256 columns of n that the token-by-token kernels keep a thread each always go this way.)
             max_chunks = n_tokens // 64 + n_entries
             scratch = torch.empty(max_chunks * heads * (d * dv + d + 3), dtype=torch.float32, device=qkvg.device)
             self._check(self.lib.ta_mlstm_chunked(_ptr(qkvg), qkvg.shape[1], _ptr(gates), gates.shape[1], _ptr(state),
