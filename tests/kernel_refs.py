@@ -39,6 +39,8 @@ class PlainOps:
         g, u = gate_up[:, :inner].to(self.work), gate_up[:, inner:].to(self.work)
         if act is None:
             out.copy_((g * torch.sigmoid(g) * u).to(out.dtype))
+        elif act == "gelu_tanh":
+            out.copy_((0.5 * g * (1.0 + torch.tanh(0.7978845608028654 * (g + 0.044715 * g * g * g))) * u).to(out.dtype))
         else:
             alpha, limit, shift = act
             g, u = torch.clamp(g, max=limit), torch.clamp(u, min=-limit, max=limit)
@@ -190,9 +192,10 @@ class PlainOps:
 
     def paged_attention(self, qkv, out, k_pages, v_pages, positions, entry_of_token, block_table,
                         n_q, n_kv, head_dim, window, scale, max_position=None, batch=None,
-                        value_dim=None, chunk=None, slopes=None, sinks=None):
+                        value_dim=None, chunk=None, slopes=None, sinks=None, keep_first=0, value_heads=None):
         page_size = k_pages.shape[2]
         group = n_q // n_kv
+        share = 1 if value_heads is None else n_kv // value_heads     # key heads that read one value head
         for t in range(qkv.shape[0]):
             if int(entry_of_token[t]) < 0:                   # a token that only fills the batch up
                 continue
@@ -201,7 +204,7 @@ class PlainOps:
             lo = max(0, pos - window) if window is not None else 0
             if chunk is not None:
                 lo = max(lo, pos // chunk * chunk)
-            keys = list(range(lo, pos + 1))
+            keys = list(range(0, min(keep_first, lo))) + list(range(lo, pos + 1))
             pages = [int(table[j // page_size]) for j in keys]
             assert all(p >= 0 for p in pages), "attention reads a page that was given back"
             offs = [j % page_size for j in keys]
@@ -209,7 +212,7 @@ class PlainOps:
             v = v_pages[pages, :, :, offs].to(self.work)      # [keys, n_kv, d]
             q = qkv[t, :n_q * head_dim].reshape(n_q, head_dim).to(self.work)
             k = k.repeat_interleave(group, dim=1)            # [keys, n_q, d]
-            v = v.repeat_interleave(group, dim=1)
+            v = v.repeat_interleave(group * share, dim=1)
             scores = torch.einsum("hd,khd->hk", q, k) * scale
             if slopes is not None:
                 distance = pos - torch.tensor(keys, dtype=self.work)
@@ -221,6 +224,100 @@ class PlainOps:
                 e = torch.exp(scores - top[:, None])
                 probs = e / (e.sum(dim=-1) + torch.exp(sinks.to(self.work) - top))[:, None]
             out[t] = torch.einsum("hk,khd->hd", probs, v).reshape(-1).to(out.dtype)
+        return out
+
+    # ------------------------------------------------------------ norms behind sub-layers, partial rotation, routing
+    def _unit(self, x, eps):
+        return x / torch.sqrt((x * x).mean(dim=-1, keepdim=True) + eps)
+
+    def norm_add_rmsnorm(self, residual, delta, post_weight, post_eps, weight, eps, out, rows=None, store_residual=True):
+        x = (residual if rows is None else residual[rows.long()]).to(self.work)
+        if delta is not None:
+            d = (delta if rows is None else delta[rows.long()]).to(self.work)
+            if post_weight is not None:
+                d = self._unit(d, post_eps) * post_weight.to(self.work)
+            x = x + d
+        if store_residual and delta is not None:
+            assert rows is None
+            residual.copy_(x.to(torch.float32))
+            x = residual.to(self.work)
+        if weight is not None:
+            x = self._unit(x, eps) * weight.to(self.work)
+        out.copy_(x.to(out.dtype))
+        return out
+
+    def norm_rotate_store(self, qkv, bias, positions, rates, dims, slots, k_pages, v_pages, n_q, n_k, n_v, d, dv,
+                          q_norm=None, k_norm=None, eps=0.0):
+        n_tokens = qkv.shape[0]
+        used = (n_q + n_k) * d + n_v * dv
+        x = qkv[:, :used].to(self.work)
+        if bias is not None:
+            x = x + bias[:used].to(self.work)
+        q, k, v = x[:, :n_q * d], x[:, n_q * d:(n_q + n_k) * d], x[:, (n_q + n_k) * d:]
+        if q_norm is not None:
+            q = self._unit(q, eps) * q_norm.to(self.work)
+        if k_norm is not None and n_k:
+            k = self._unit(k, eps) * k_norm.to(self.work)
+        turn = torch.cat([q, k], dim=1).reshape(n_tokens, n_q + n_k, d).clone()
+        half = dims // 2
+        if half:
+            angles = positions.to(torch.float32)[:, None] * rates.to(torch.float32)[None, :]      # float32 angles
+            cos, sin = angles.cos().to(self.work)[:, None, :], angles.sin().to(self.work)[:, None, :]
+            a, b = turn[..., :half].clone(), turn[..., half:dims].clone()
+            turn[..., :half] = a * cos - b * sin
+            turn[..., half:dims] = b * cos + a * sin
+        qkv[:, :used] = torch.cat([turn.reshape(n_tokens, -1), v], dim=1).to(qkv.dtype)
+        if slots is not None:
+            page_size = k_pages.shape[2]
+            keys = qkv[:, n_q * d:(n_q + n_k) * d].reshape(n_tokens, n_k, d)
+            values = qkv[:, (n_q + n_k) * d:used].reshape(n_tokens, n_v, dv)
+            for t in range(n_tokens):
+                slot = int(slots[t])
+                if slot < 0:
+                    continue
+                page, off = divmod(slot, page_size)
+                k_pages[page, :, off, :] = keys[t]
+                v_pages[page, :, :, off] = values[t]
+
+    def differential_heads(self, mixed, lam, eps, out_scale, n_heads, group, dv, out):
+        n_tokens = mixed.shape[0]
+        maps = mixed.to(self.work).reshape(n_tokens, n_heads // group, 2, group, dv)
+        o = maps[:, :, 0] - lam.to(self.work).reshape(()) * maps[:, :, 1]            # [T, kv heads, group, dv]
+        out.copy_((self._unit(o, eps) * out_scale).reshape(n_tokens, n_heads * dv).to(out.dtype))
+        return out
+
+    def sigmoid_head_gate(self, mixed, rows, offset, n_heads, dv):
+        gate = torch.sigmoid(rows[:, offset:offset + n_heads].to(self.work))
+        x = mixed.to(self.work).reshape(mixed.shape[0], n_heads, dv) * gate[:, :, None]
+        mixed.copy_(x.reshape(mixed.shape).to(mixed.dtype))
+        return mixed
+
+    def side_gate(self, gate, table, token_ids, offset, dim, out):
+        g = gate.to(self.work)
+        act = 0.5 * g * (1.0 + torch.tanh(0.7978845608028654 * (g + 0.044715 * g * g * g)))
+        e = torch.zeros_like(act)
+        e[:, :dim] = table[token_ids.long()][:, offset:offset + dim].to(self.work)
+        out.copy_((act * e).to(out.dtype))
+        return out
+
+    def route_top(self, logits, chosen, weights):
+        top = chosen.shape[1]
+        values, ids = torch.topk(logits.to(torch.float32), top, dim=-1)
+        chosen.copy_(ids.to(torch.int32))
+        weights.copy_(torch.softmax(values, dim=-1))
+
+    def expert_gate(self, gate_up, chosen, weights, n_experts, inner, shared, out):
+        n_tokens = gate_up.shape[0]
+        x = gate_up.to(self.work)
+        out.zero_()
+        routed = x[:, :n_experts * 2 * inner].reshape(n_tokens, n_experts, 2, inner)
+        factor = torch.zeros((n_tokens, n_experts), dtype=self.work)
+        factor.scatter_(1, chosen.long(), weights.to(self.work))
+        g, u = routed[:, :, 0], routed[:, :, 1]
+        out[:, :n_experts * inner] = (factor[:, :, None] * (g * torch.sigmoid(g) * u)).reshape(n_tokens, -1).to(out.dtype)
+        if shared:
+            g, u = x[:, n_experts * 2 * inner:n_experts * 2 * inner + shared], x[:, n_experts * 2 * inner + shared:]
+            out[:, n_experts * inner:n_experts * inner + shared] = (g * torch.sigmoid(g) * u).to(out.dtype)
         return out
 
     def linear(self, x, weight, bias=None, out=None, out_dtype=None):

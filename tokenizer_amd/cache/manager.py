@@ -155,6 +155,9 @@ class CacheManager:
         if not self._core:
             raise ValueError("num_pages and max_requests must not be negative and page_size must be positive")
         self._core_owner = _CoreOwner(self._lib, self._core)
+        for g, (need, _) in enumerate(planned):
+            if need.keep_first:              # the first positions stay readable behind the window
+                self._lib.ta_cache_set_keep_first(self._core, g, int(need.keep_first))
         self.groups = [CacheGroup(need, layers, PageAllocator(num_pages, page_size,
                                                               _borrowed=self._lib.ta_cache_allocator(self._core, g),
                                                               _owner=self._core_owner))

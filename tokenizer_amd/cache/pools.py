@@ -27,8 +27,9 @@ class CachePools:
                 raise ValueError(f"{manager.num_pages} pages of {manager.page_size} tokens are {per_layer} key elements "
                                  f"a layer; the kernels address fewer than 2^31 (at most "
                                  f"{(2 ** 31 - 1) // (need.n_kv_heads * manager.page_size * max(need.head_dim, need.v_dim))} pages here)")
-            self.pages.append(torch.zeros((len(group.layers), manager.num_pages * need.n_kv_heads * manager.page_size
-                                           * (need.head_dim + need.v_dim)), dtype=dtype, device=device))
+            self.pages.append(torch.zeros((len(group.layers), manager.num_pages * manager.page_size
+                                           * (need.n_kv_heads * need.head_dim + need.v_heads * need.v_dim)),
+                                          dtype=dtype, device=device))
         self.states, self.block_states = {}, {}
         for layer, need in enumerate(needs):
             if need.state_shape is not None:
@@ -39,8 +40,8 @@ class CachePools:
                                                        dtype=torch.float32, device=device)
 
     def layer_pages(self, layer: int):
-        """(keys [num_pages, n_kv, page_size, d], values [num_pages, n_kv, dv, page_size]) of one layer,
-        or (None, None)."""
+        """(keys [num_pages, n_kv, page_size, d], values [num_pages, n_v, dv, page_size]) of one layer (n_v = n_kv
+        unless the need names fewer value heads), or (None, None)."""
         group = self.manager.group_of_layer[layer]
         if group is None:
             return None, None
@@ -50,7 +51,7 @@ class CachePools:
         shape = (self.manager.num_pages, need.n_kv_heads)
         keys = shape[0] * shape[1] * page_size * need.head_dim
         return (pages[index, :keys].view(*shape, page_size, need.head_dim),
-                pages[index, keys:].view(*shape, need.v_dim, page_size))
+                pages[index, keys:].view(shape[0], need.v_heads, need.v_dim, page_size))
 
     def keep_states(self) -> list:
         """Copies of every state tensor (for a run whose effect on them is to be undone)."""

@@ -3,7 +3,8 @@ from .registry import (Architecture, architecture_name, get_architecture, load_c
                        register_architecture, registered_architectures)
 from .qwen2 import Qwen2Config
 from .napadra import NapadraConfig
+from .dolidra import DolidraConfig
 
 __all__ = ["ConfigError", "ModelConfig", "read_config_json", "Architecture", "architecture_name",
            "get_architecture", "load_config", "register_architecture", "registered_architectures",
-           "Qwen2Config", "NapadraConfig"]
+           "Qwen2Config", "NapadraConfig", "DolidraConfig"]

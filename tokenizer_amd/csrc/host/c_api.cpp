@@ -97,6 +97,12 @@ void* ta_cache_new(int n_groups, const int* windows, int num_pages, int page_siz
   if (n_groups < 0 || num_pages < 0 || page_size <= 0 || max_requests < 0 || n_state_layers < 0) return nullptr;
   return new CacheCore(n_groups, windows, num_pages, page_size, max_requests, prefix_cache != 0, n_state_layers);
 }
+// The first `count` positions of every sequence stay readable in group `group` (their pages are never given back).
+int ta_cache_set_keep_first(void* c, int group, int count) {
+  if (group < 0 || group >= ((CacheCore*)c)->n_groups()) return -1;
+  ((CacheCore*)c)->set_keep_first(group, count);
+  return 0;
+}
 void ta_cache_delete(void* c) { delete (CacheCore*)c; }
 void* ta_cache_allocator(void* c, int group) { return ((CacheCore*)c)->allocator(group); }   // borrowed
 int ta_cache_prefix_enabled(void* c) { return ((CacheCore*)c)->prefix_cache() ? 1 : 0; }

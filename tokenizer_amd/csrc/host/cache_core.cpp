@@ -94,7 +94,7 @@ int CacheCore::advance(int64_t id, int new_len) {
     // Pages no later query reads again go back to the pool.
     const int first = first_needed_position((int)g, new_len);
     std::vector<int>& table = request->tables[g];
-    for (int index = 0; index < first / page_size_; ++index) {
+    for (int index = pages_for_len(groups_[g]->keep_first, page_size_); index < first / page_size_; ++index) {
       if (table[index] >= 0) {
         groups_[g]->allocator.free_page(table[index], nullptr);
         table[index] = -1;

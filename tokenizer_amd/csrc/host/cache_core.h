@@ -21,8 +21,11 @@ enum CacheStatus {
 // A group of layers with one need: `window` < 0 keeps the keys of every position; a window w >= 0 means that a
 // query reads the keys at most w positions behind it, so pages wholly behind every later query are given back.
 // (Whatever a mixer calls its kind of cache, it reaches this class as that one number.)
+// `keep_first` > 0: the pages that hold the first so many positions of a sequence stay with the request whatever
+// the window says (queries go on reading those positions).
 struct Group {
   int window;
+  int keep_first = 0;
   PageAllocator allocator;
   bool keeps_all() const { return window < 0; }
   Group(int window, int num_pages, int page_size) : window(window), allocator(num_pages, page_size) {}
@@ -41,6 +44,8 @@ class CacheCore {
   // positions and no layer keeps such state (a state slot has seen every token; an attached prefix would skip them).
   CacheCore(int n_groups, const int* windows, int num_pages, int page_size, int max_requests, bool prefix_cache,
             int n_state_layers);
+
+  void set_keep_first(int group, int count) { groups_[group]->keep_first = count < 0 ? 0 : count; }
 
   int n_groups() const { return (int)groups_.size(); }
   int page_size() const { return page_size_; }

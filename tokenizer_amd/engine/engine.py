@@ -258,11 +258,12 @@ class Engine:
         self.pools = CachePools(self.cache, model.cache_needs, model.dtype, model.device)
         self.layer_caches = []
         for entry in model.spec.schedule:
-            source = entry.layer if entry.cache_of is None else entry.cache_of
+            source = entry.cache_unit()          # the layer's own unit, another layer's, or this run's own
             k_pages, v_pages = self.pools.layer_pages(source)
             self.layer_caches.append(LayerCache(group=self.cache.group_of_layer[source], k_pages=k_pages,
                                                 v_pages=v_pages, state=self.pools.states.get(source),
-                                                block_state=self.pools.block_states.get(entry.layer),
+                                                block_state=self.pools.block_states.get(
+                                                    entry.layer if entry.unit is None else entry.unit),
                                                 writes=entry.cache_of is None))
         self.steps = 0
         self._landing: dict[int, tuple] = {}     # pinned rows and events of `decode_greedy` / `decode_sampled`, by batch size

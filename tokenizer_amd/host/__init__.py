@@ -34,6 +34,7 @@ _SIGNATURES = {
     "ta_alloc_reclaim_cached": (None, [_vp]),
     "ta_alloc_check": (_int, [_vp]),
     "ta_cache_new": (_vp, [_int, _i32p, _int, _int, _int, _int, _int]),
+    "ta_cache_set_keep_first": (_int, [_vp, _int, _int]),
     "ta_cache_delete": (None, [_vp]),
     "ta_cache_allocator": (_vp, [_vp, _int]),
     "ta_cache_prefix_enabled": (_int, [_vp]),

@@ -1,2 +1,3 @@
 from . import qwen2  # noqa: F401  (registers Qwen2ForCausalLM)
 from . import napadra  # noqa: F401  (registers Napadra)
+from . import dolidra  # noqa: F401  (registers Dolidra)

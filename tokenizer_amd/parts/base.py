@@ -190,6 +190,21 @@ class Block:
         raise NotImplementedError
 
 
+class NormedDelta:
+    """What a sub-layer that is normalised behind itself hands on: its output `rows` [T, H] (compute dtype) still to
+    be brought to unit RMS, scaled by `weight` (float32 [H]) and added to the stream.  A norm of the form
+    x / sqrt(mean(x^2) + eps) * w takes it as its delta and does all of that in its own kernel
+    (`ops.norm_add_rmsnorm`); for anyone else `resolve()` gives the sum's term as a float32 tensor."""
+
+    def __init__(self, ops, rows: torch.Tensor, weight: torch.Tensor, eps: float):
+        self.ops, self.rows, self.weight, self.eps = ops, rows, weight, float(eps)
+
+    def resolve(self) -> torch.Tensor:
+        zero = torch.zeros((self.rows.shape[0], self.rows.shape[1]), dtype=torch.float32, device=self.rows.device)
+        out = torch.empty_like(zero)
+        return self.ops.norm_add_rmsnorm(zero, self.rows, self.weight, self.eps, None, 0.0, out, store_residual=False)
+
+
 def as_tensor(delta):
     """The delta as a tensor: a product still in parts has them added now."""
     resolve = getattr(delta, "resolve", None)

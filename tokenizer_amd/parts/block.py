@@ -1,7 +1,10 @@
 """Arrangements of norms, mixer and feed-forward around the residual stream."""
 from __future__ import annotations
 
-from .base import BLOCKS, Block, Repeatable, repeatable_of
+import torch
+
+from .base import BLOCKS, Block, NormedDelta, Repeatable, as_tensor, repeatable_of
+from .spec import TensorSpec
 
 
 @BLOCKS.register("pre_norm")
@@ -32,4 +35,74 @@ class PreNormBlock(Block):
             delta = self.mixer.forward_normed(residual, delta, self.mixer_norm, ctx, cache)
         if self.feed_forward is not None:
             delta = self.feed_forward.forward_normed(residual, delta, self.feed_forward_norm, ctx)
+        return delta
+
+
+@BLOCKS.register("sandwich_norm")
+class SandwichNormBlock(Block):
+    """x + norm_b(mixer(norm(x))), then + norm_b'(feed_forward(norm'(.))): every sub-layer is normalised before and
+    behind (RMS norms with weights; the ones behind are the block's own tensors `norm1b`, `norm2b`), and behind the
+    feed-forward the layer may add an input made from the token itself (option `side_dim` > 0): with e the layer's
+    slice [side_offset, side_offset + side_dim) of the token's row in the shared table `side_table`,
+    y = proj(gelu_tanh(gate x) * e), x + y / sqrt(mean(y^2) + eps) * side.norm (tensors `side.gate` [side_dim, width],
+    `side.proj` [width, side_dim], `side.norm` [width]).
+
+    The stream is float32.  A sub-layer's output is handed on as a `NormedDelta`: the norm that takes it next brings
+    it to unit RMS, scales it, adds it to the stream and normalises the sum in one kernel.
+    """
+    graph_safe = True
+
+    @staticmethod
+    def tensor_specs(layer) -> dict:
+        width, out = int(layer.options["width"]), {}
+        if layer.mixer is not None:
+            out["norm1b"] = TensorSpec((width,), init="ones", role="vector")
+        if layer.feed_forward is not None:
+            out["norm2b"] = TensorSpec((width,), init="ones", role="vector")
+        side = int(layer.options.get("side_dim") or 0)
+        if side:
+            out.update({"side.gate": TensorSpec((side, width)), "side.proj": TensorSpec((width, side)),
+                        "side.norm": TensorSpec((width,), init="ones", role="vector"),
+                        "/" + layer.options["side_table"]: TensorSpec((int(layer.options["vocab"]),
+                                                                       int(layer.options["side_width"])))})
+        return out
+
+    def __init__(self, mixer_norm, mixer, feed_forward_norm, feed_forward, layer, tensors, runtime):
+        self.mixer_norm, self.mixer = mixer_norm, mixer
+        self.feed_forward_norm, self.feed_forward = feed_forward_norm, feed_forward
+        self.runtime, self.eps = runtime, float(layer.options["eps"])
+        self.width = int(layer.options["width"])
+        self.after_mixer = tensors["norm1b"] if mixer is not None else None
+        self.after_feed_forward = tensors["norm2b"] if feed_forward is not None else None
+        self.side_dim = int(layer.options.get("side_dim") or 0)
+        if self.side_dim:
+            self.side_offset = int(layer.options["side_offset"])
+            self.side_table = tensors["/" + layer.options["side_table"]]
+            self.side_gate, self.side_proj, self.side_norm = tensors["side.gate"], tensors["side.proj"], tensors["side.norm"]
+            # The bfloat16 products read eight elements of K at a time: a narrower token input is filled up with
+            # zero rows of the gate and zero columns of the projection.
+            fill = (-self.side_dim) % 8 if runtime.dtype == torch.bfloat16 else 0
+            if fill:
+                self.side_gate = torch.cat([self.side_gate, self.side_gate.new_zeros((fill, self.width))], dim=0).contiguous()
+                self.side_proj = torch.cat([self.side_proj, self.side_proj.new_zeros((self.width, fill))], dim=1).contiguous()
+
+    def forward(self, residual, delta, ctx, cache):
+        ops = self.runtime.ops
+        if self.mixer is not None:
+            mixed = self.mixer.forward(self.mixer_norm.apply(residual, delta), ctx, cache)
+            delta = NormedDelta(ops, mixed, self.after_mixer, self.eps)
+        if self.feed_forward is not None:
+            out = self.feed_forward.forward(self.feed_forward_norm.apply(residual, delta), ctx)
+            delta = NormedDelta(ops, out, self.after_feed_forward, self.eps)
+        if self.side_dim:
+            # The stream as it stands behind the feed-forward, in the compute dtype, for the gate's product.
+            rows = torch.empty((residual.shape[0], self.width), dtype=self.runtime.dtype, device=residual.device)
+            if isinstance(delta, NormedDelta):
+                ops.norm_add_rmsnorm(residual, delta.rows, delta.weight, delta.eps, None, 0.0, rows)
+            else:                                   # what a block of another kind handed on: a plain sum, or nothing
+                ops.norm_add_rmsnorm(residual, None if delta is None else as_tensor(delta), None, 0.0, None, 0.0, rows)
+            gate = ops.linear(rows, self.side_gate)
+            gated = torch.empty_like(gate)
+            ops.side_gate(gate, self.side_table, ctx.token_ids, self.side_offset, self.side_dim, gated)
+            delta = NormedDelta(ops, ops.linear(gated, self.side_proj), self.side_norm, self.eps)
         return delta

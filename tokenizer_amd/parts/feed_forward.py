@@ -19,9 +19,10 @@ class GatedDense(FeedForward):
 
 
     def __init__(self, spec: FeedForwardSpec, tensors: dict[str, torch.Tensor], runtime: Runtime):
-        if spec.activation not in ("silu", "capped_swish"):
-            raise ValueError(f"gated_dense knows the activations silu and capped_swish, not {spec.activation!r}")
+        if spec.activation not in ("silu", "capped_swish", "gelu_tanh"):
+            raise ValueError(f"gated_dense knows the activations silu, gelu_tanh and capped_swish, not {spec.activation!r}")
         self.spec, self.runtime = spec, runtime
+        self.gelu = spec.activation == "gelu_tanh"     # 0.5 g (1 + tanh(sqrt(2/pi) (g + 0.044715 g^3))) in place of silu
         # capped_swish: g' = min(g, limit), u' = clamp(u, -limit, limit); g' * sigmoid(alpha g') * (u' + shift).
         # (silu is alpha 1, no limit, shift 0, and keeps the kernels written for it.)
         self.act = None
@@ -48,6 +49,8 @@ class GatedDense(FeedForward):
                 "down_proj.weight": TensorSpec((spec.hidden_size, spec.intermediate_size))}
 
     def repeatable(self):
+        if self.gelu:
+            return None
         return Repeatable(("gated_dense", self.act), (self.w_gate_up, self.w_down))
 
     def forward_normed(self, residual, delta, norm, ctx):
@@ -55,7 +58,7 @@ class GatedDense(FeedForward):
         down product added straight into the residual stream."""
         ops = self.runtime.ops
         fold = norm.fold() if delta is None else None      # the norm says whether it has the form the kernel computes
-        if fold is None or self.act is not None or not _can_fuse(ops, residual, self.runtime.dtype):
+        if fold is None or self.act is not None or self.gelu or not _can_fuse(ops, residual, self.runtime.dtype):
             # The output is handed on as a delta: a down product whose K is cut over workgroups may stay in
             # parts, and the norm that takes it next adds them in its own kernel.
             return self._run(norm.apply(residual, delta), pending=getattr(ops, "takes_pending", False))
@@ -71,7 +74,9 @@ class GatedDense(FeedForward):
 
     def _run(self, x, pending: bool):
         ops = self.runtime.ops
-        if self.act is None:
+        if self.gelu:
+            act = ops.linear_silu_gate(x, self.w_gate_up, act="gelu_tanh")
+        elif self.act is None:
             act = ops.linear_silu_gate(x, self.w_gate_up)
         elif _can_fuse(ops, x, self.runtime.dtype) and x.shape[1] % 8 == 0:
             # Up to sixteen normalised rows: the fused decode product with the capped activation in its epilogue.
@@ -79,3 +84,63 @@ class GatedDense(FeedForward):
         else:
             act = ops.linear_silu_gate(x, self.w_gate_up, act=self.act)
         return ops.linear(act, self.w_down, pending=True) if pending else ops.linear(act, self.w_down)
+
+
+@FEED_FORWARDS.register("routed_experts")
+class RoutedExperts(FeedForward):
+    """A mixture of `n_experts` small gated feed-forwards (tensors `e<j>.gate|up|down`, inner width
+    `intermediate_size`, silu, no biases), of which every token uses the `top_k` with the largest router logits
+    (`router` [n_experts, hidden]; the logits are float32 sums), weighted by the softmax over the chosen logits alone;
+    an optional shared expert (`shared.gate|up|down`, inner width `shared_size`) runs for every token and is added.
+
+    All experts' gate and up matrices are one matrix, and all down matrices one matrix along K, so a step is two
+    products whatever the routing: between them a kernel turns gate and up into weight * silu(gate) * up for the
+    experts a token chose and into zero for the others (the shared expert counts as chosen with weight 1), and the
+    second product then adds the chosen experts' outputs up in its own sum.  The routing stays on the device, so
+    the step's launches do not depend on it.
+    """
+    graph_safe = True
+
+    def __init__(self, spec: FeedForwardSpec, tensors: dict[str, torch.Tensor], runtime: Runtime):
+        if spec.activation != "silu":
+            raise ValueError(f"routed_experts knows the activation silu, not {spec.activation!r}")
+        if not 0 < spec.top_k <= spec.n_experts:
+            raise ValueError(f"{spec.top_k} of {spec.n_experts} experts")
+        self.spec, self.runtime = spec, runtime
+        self.n_experts, self.top_k = spec.n_experts, spec.top_k
+        self.inner, self.shared = spec.intermediate_size, spec.shared_size
+        self.w_router = tensors["router"]
+        names = [f"e{j}" for j in range(self.n_experts)] + (["shared"] if self.shared else [])
+        gate_up, down = [], []
+        for name in names:
+            gate_up += [tensors[f"{name}.gate"], tensors[f"{name}.up"]]
+            down.append(tensors[f"{name}.down"])
+        self.total = self.n_experts * self.inner + self.shared           # columns between the two products
+        fill = (-self.total) % 8 if runtime.dtype == torch.bfloat16 else 0     # the second product reads K in eights
+        if fill:
+            down.append(down[0].new_zeros((spec.hidden_size, fill)))
+        self.w_gate_up = torch.cat(gate_up, dim=0).contiguous()
+        self.w_down = torch.cat(down, dim=1).contiguous()
+        self.columns = self.total + fill
+
+    @staticmethod
+    def tensor_specs(spec: FeedForwardSpec) -> dict[str, TensorSpec]:
+        out = {"router": TensorSpec((spec.n_experts, spec.hidden_size), std=0.5)}
+        sizes = [(f"e{j}", spec.intermediate_size) for j in range(spec.n_experts)]
+        if spec.shared_size:
+            sizes.append(("shared", spec.shared_size))
+        for name, inner in sizes:
+            out.update({f"{name}.gate": TensorSpec((inner, spec.hidden_size)), f"{name}.up": TensorSpec((inner, spec.hidden_size)),
+                        f"{name}.down": TensorSpec((spec.hidden_size, inner))})
+        return out
+
+    def forward(self, x, ctx):
+        ops = self.runtime.ops
+        logits = ops.linear(x, self.w_router, out_dtype=torch.float32)
+        chosen = torch.empty((x.shape[0], self.top_k), dtype=torch.int32, device=x.device)
+        weights = torch.empty((x.shape[0], self.top_k), dtype=torch.float32, device=x.device)
+        ops.route_top(logits, chosen, weights)
+        gate_up = ops.linear(x, self.w_gate_up)
+        act = torch.empty((x.shape[0], self.columns), dtype=x.dtype, device=x.device)
+        ops.expert_gate(gate_up, chosen, weights, self.n_experts, self.inner, self.shared, act)
+        return ops.linear(act, self.w_down)

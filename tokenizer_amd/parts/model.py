@@ -10,8 +10,10 @@ from .spec import CacheNeed, ModelSpec, TensorSpec
 
 
 def _prefixed(prefix: str, specs: dict[str, TensorSpec]) -> dict[str, TensorSpec]:
-    """(A part's tensor with the empty name is the tensor that the prefix itself names.)"""
-    return {(f"{prefix}.{name}" if name else prefix) if prefix else name: spec for name, spec in specs.items()}
+    """(A part's tensor with the empty name is the tensor that the prefix itself names; a name that starts with "/"
+    is the model's own, whatever the prefix: a table that several layers share.)"""
+    return {name[1:] if name.startswith("/") else (f"{prefix}.{name}" if name else prefix) if prefix else name: spec
+            for name, spec in specs.items()}
 
 
 def _renamed(specs: dict[str, TensorSpec], names) -> dict[str, TensorSpec]:
@@ -31,8 +33,10 @@ def expected_tensors(spec: ModelSpec) -> dict[str, TensorSpec]:
 
 
 def cache_needs(spec: ModelSpec) -> list[CacheNeed]:
-    """What each layer asks of the cache manager, by layer index: the model's frame says."""
-    return FRAMES.get(spec.frame).cache_needs(spec)
+    """What each cache unit asks of the cache manager: the layers' own units by layer index, as the model's frame
+    says, then the further units of runs that keep a cache of their own (`ModelSpec.extra_cache_units`)."""
+    needs = list(FRAMES.get(spec.frame).cache_needs(spec))
+    return needs + [needs[layer] for layer in spec.extra_cache_units]
 
 
 def build_model(spec: ModelSpec, tensors: dict[str, torch.Tensor], runtime: Runtime):
@@ -46,6 +50,14 @@ def _strip(prefix: str, tensors: dict[str, torch.Tensor]) -> dict[str, torch.Ten
     if prefix in tensors:
         out[""] = tensors[prefix]
     return out
+
+
+def _with_shared(own: dict[str, torch.Tensor], wanted, tensors: dict[str, torch.Tensor]) -> dict[str, torch.Tensor]:
+    """A part's tensors with the model's own that it asked for by a name starting with "/"."""
+    for name in wanted:
+        if name.startswith("/"):
+            own[name] = tensors[name[1:]]
+    return own
 
 
 @dataclasses.dataclass
@@ -189,7 +201,8 @@ class DecoderModel:
             block = BLOCKS.get(layer.block)
             if hasattr(block, "tensor_specs"):     # a block with tensors and constants of its own is handed them
                 self.blocks.append(block(mixer_norm, mixer, ff_norm, feed_forward, layer=layer,
-                                         tensors=_strip(layer.prefix, tensors), runtime=runtime))
+                                         tensors=_with_shared(_strip(layer.prefix, tensors), block.tensor_specs(layer), tensors),
+                                         runtime=runtime))
             else:
                 self.blocks.append(block(mixer_norm, mixer, ff_norm, feed_forward))
         self.final_norm = NORMS.get(spec.final_norm.kind)(spec.final_norm, _strip(spec.final_norm_prefix, tensors), runtime)

@@ -3,24 +3,27 @@ from __future__ import annotations
 
 import torch
 
-from .base import NORMS, Norm, NormFold, Repeatable, Runtime
+from .base import NORMS, Norm, NormedDelta, NormFold, Repeatable, Runtime
 from .spec import NormSpec, TensorSpec
 
 
 @NORMS.register("rmsnorm")
 class RMSNorm(Norm):
-    """y = x / sqrt(mean(x^2) + eps) * weight (qwen-infer/src/model.rs:594-599), in float32."""
+    """y = x / sqrt(mean(x^2) + eps) * weight (qwen-infer/src/model.rs:594-599), in float32.  The weight is the
+    tensor `weight` under the norm's prefix, or (option `tensor_name`) another name there; the empty name is the
+    tensor that the prefix itself names.  A delta that is itself still to be normalised (`NormedDelta`) is
+    normalised, scaled and added in the same kernel."""
     graph_safe = True
 
 
     def __init__(self, spec: NormSpec, tensors: dict[str, torch.Tensor], runtime: Runtime):
         self.size, self.eps = spec.size, float(spec.eps)
-        self.weight = tensors["weight"]
+        self.weight = tensors[spec.options.get("tensor_name", "weight")]
         self.runtime = runtime
 
     @staticmethod
     def tensor_specs(spec: NormSpec) -> dict[str, TensorSpec]:
-        return {"weight": TensorSpec((spec.size,), init="ones", role="vector")}
+        return {spec.options.get("tensor_name", "weight"): TensorSpec((spec.size,), init="ones", role="vector")}
 
     def fold(self):
         return NormFold(self.weight, self.eps)
@@ -31,6 +34,9 @@ class RMSNorm(Norm):
     def apply(self, residual, delta, rows=None):
         n_rows = residual.shape[0] if rows is None else rows.numel()
         out = torch.empty((n_rows, self.size), dtype=self.runtime.dtype, device=residual.device)
+        if isinstance(delta, NormedDelta):
+            return self.runtime.ops.norm_add_rmsnorm(residual, delta.rows, delta.weight, delta.eps, self.weight, self.eps,
+                                                     out, rows, store_residual=rows is None)
         return self.runtime.ops.add_rmsnorm(residual, delta, self.weight, self.eps, out, rows,
                                             store_residual=rows is None)
 

@@ -1,6 +1,8 @@
 """Position encodings applied to queries and keys before the keys go into the cache."""
 from __future__ import annotations
 
+import math
+
 import torch
 
 from .base import POSITIONS, PositionEncoding, Repeatable, Runtime, StoreEpilogue
@@ -72,3 +74,54 @@ class RotaryHalfSplit(NoPosition):
 
     def repeatable(self):
         return Repeatable(("rope_half_split", self.max_positions), (self.cos_sin,))
+
+
+def scaled_rates(theta: float, dims: int, scaling: dict | None) -> torch.Tensor:
+    """float32 [dims / 2]: the rates f_i = theta^(-2i/dims), worked out in float64.  `scaling` (factor, low, high,
+    original) slows the long waves: with wavelength l = 2 pi / f a rate stays as it is where l < original / high,
+    becomes f / factor where l > original / low, and in between is (1 - s) f / factor + s f with
+    s = (original / l - low) / (high - low)."""
+    rates = []
+    for i in range(dims // 2):
+        f = float(theta) ** (-2.0 * i / dims)
+        if scaling:
+            factor, low, high, original = (float(scaling[key]) for key in ("factor", "low", "high", "original"))
+            wave = 2.0 * math.pi / f
+            if wave > original / low:
+                f = f / factor
+            elif wave >= original / high:
+                s = (original / wave - low) / (high - low)
+                f = (1.0 - s) * f / factor + s * f
+        rates.append(f)
+    return torch.tensor(rates, dtype=torch.float64).to(torch.float32)
+
+
+@POSITIONS.register("rope_partial")
+class RotaryPartial(PositionEncoding):
+    """Rotation of the first `dims` coordinates of every query and key head (options `dims`, even and at most the
+    head size; `scaling`, see `scaled_rates`): coordinate i < dims / 2 is paired with coordinate i + dims / 2 and the
+    pair turns by the angle position * f_i; the coordinates from `dims` on pass unchanged.  There is no table of
+    positions: the kernel forms the angle in float32 from the position and the rate and takes its accurate sine and
+    cosine, so positions are bounded by nothing here.  Keys are stored after the rotation.
+
+    The same kernel adds the projection's bias before and, for mixers that ask for it, normalises all query rows
+    at once and all key rows at once (an RMS norm with a weight over the whole projection) before the rotation."""
+    graph_safe = True
+
+    def __init__(self, spec: PositionSpec, runtime: Runtime):
+        self.runtime = runtime
+        self.dims = int(spec.options.get("dims", spec.head_dim))
+        if self.dims % 2 or not 0 <= self.dims <= spec.head_dim:
+            raise ValueError(f"a rotation over {self.dims} of {spec.head_dim} coordinates")
+        self.rates = scaled_rates(spec.theta, self.dims, spec.options.get("scaling")).to(runtime.device).contiguous()
+
+    def encode_and_store(self, qkv, bias, n_q, n_kv, head_dim, ctx, cache, value_dim=None, value_heads=None,
+                         q_norm=None, k_norm=None, eps=0.0):
+        """Rows of `qkv`: n_q query heads and n_kv key heads of `head_dim`, then `value_heads` (n_kv if None) value
+        heads of `value_dim`; whatever lies behind them in a row is left alone."""
+        slots = ctx.slots[cache.group] if cache.writes and n_kv else None
+        self.runtime.ops.norm_rotate_store(qkv, bias, ctx.positions, self.rates, self.dims, slots,
+                                           cache.k_pages if slots is not None else None,
+                                           cache.v_pages if slots is not None else None, n_q, n_kv,
+                                           n_kv if value_heads is None else value_heads, head_dim,
+                                           head_dim if value_dim is None else value_dim, q_norm, k_norm, eps)

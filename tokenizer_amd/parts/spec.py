@@ -40,6 +40,9 @@ class CacheNeed:
     `value_dim`: size of a value head where it differs from the key heads' `head_dim` (0: the same).
     `block_state_shape`: per-request state that the block around the mixer keeps in the same slot (the last
     token's normalised row, for a token shift), or None; always float32.
+    `keep_first`: with a window, the first so many positions of a sequence stay readable for every later query.
+    `n_value_heads`: the number of value heads where it is not the number of key heads (several key heads, the
+    maps of one differential head, read the same values).
     """
     kind: str = "none"
     n_kv_heads: int = 0
@@ -49,14 +52,20 @@ class CacheNeed:
     state_dtype: str = "float32"
     value_dim: int = 0
     block_state_shape: tuple[int, ...] | None = None
+    keep_first: int = 0           # kind "window": the pages of the first so many positions are never given back
+    n_value_heads: int = 0        # value heads where several key heads read one value head (0: as many as key heads)
 
     @property
     def v_dim(self) -> int:
         return self.value_dim or self.head_dim
 
+    @property
+    def v_heads(self) -> int:
+        return self.n_value_heads or self.n_kv_heads
+
     def page_key(self) -> tuple:
         """Layers with equal keys share one group of pages and one block table."""
-        return (self.kind, self.n_kv_heads, self.head_dim, self.window, self.v_dim)
+        return (self.kind, self.n_kv_heads, self.head_dim, self.window, self.v_dim, self.keep_first, self.v_heads)
 
 
 @dataclasses.dataclass(frozen=True)
@@ -96,6 +105,11 @@ class MixerSpec:
     own_kv: bool = True           # False: no key/value projections; the layer reads the cache it is pointed at
     gate_cap: float | None = None  # recurrent mixers: the cap on the gates' pre-activations
     eps: float = 0.0              # mixers with a norm of their own inside
+    keep_first: int = 0           # with a window: keys at positions below this stay visible to every later query
+    differential: float | None = None   # c: two score maps per head over the same values, o = a1 - lambda a2 with
+    #                               lambda = exp(lq1.lk1) - exp(lq2.lk2) + c, o brought to unit RMS per head, times 1 - c
+    qk_norm: str | None = None    # "whole": RMS norm with a weight over all query rows at once (and all key rows), before rotation
+    head_gate: bool = False       # each head's output times sigmoid of one number projected from the mixer's input
     tensor_names: tuple[tuple[str, str], ...] = ()   # (part's name, file's name) where a file names tensors otherwise
     options: dict[str, Any] = dataclasses.field(default_factory=dict, hash=False, compare=False)
 
@@ -105,10 +119,13 @@ class FeedForwardSpec:
     kind: str                     # "gated_dense", ...
     hidden_size: int
     intermediate_size: int = 0
-    activation: str = "silu"      # "silu", or "capped_swish" with the three numbers below
+    activation: str = "silu"      # "silu", "gelu_tanh", or "capped_swish" with the three numbers below
     act_alpha: float = 1.0        # g * sigmoid(alpha g)
     act_limit: float | None = None  # g is cut at +limit, the other branch at +-limit
     act_up_shift: float = 0.0     # added to the other branch before the product
+    n_experts: int = 0            # routed feed-forwards: experts of `intermediate_size`, of which a token uses `top_k`
+    top_k: int = 0
+    shared_size: int = 0          # inner width of an expert that every token uses (0: none)
     tensor_names: tuple[tuple[str, str], ...] = ()
     options: dict[str, Any] = dataclasses.field(default_factory=dict, hash=False, compare=False)
 
@@ -146,10 +163,19 @@ class LayerSpec:
 class ScheduleEntry:
     """Run `layer`; its mixer uses the cache of `cache_of` (default: its own).
 
-    A layer that reads another layer's cache writes nothing into it.
+    A layer that reads another layer's cache writes nothing into it.  `unit`: the run has a cache of its own under
+    this number instead of the layer's (a layer that runs several times with the same weights and keeps keys,
+    values and state of each run apart): units 0..n_layers-1 are the layers' own, `ModelSpec.extra_cache_units`
+    lists the further ones, each by the layer whose need it repeats.
     """
     layer: int
     cache_of: int | None = None
+    unit: int | None = None
+
+    def cache_unit(self) -> int:
+        if self.unit is not None:
+            return self.unit
+        return self.layer if self.cache_of is None else self.cache_of
 
 
 @dataclasses.dataclass(frozen=True)
@@ -167,4 +193,5 @@ class ModelSpec:
     head_name: str                # used when the head is not tied
     embedding_std: float = 0.02
     frame: str = "decoder"        # what stands around the layers (`parts.base.FRAMES`)
+    extra_cache_units: tuple[int, ...] = ()   # cache unit n_layers + i repeats the need of layer extra_cache_units[i]
     options: dict[str, Any] = dataclasses.field(default_factory=dict, hash=False, compare=False)   # the frame's own constants
