@@ -13,6 +13,8 @@
 // chunk > 0: only keys of the query's own run of `chunk` positions (runs counted from position 0) are seen.
 // slopes (float [n_q] or null): head h's score loses slopes[h] for every position between query and key.
 // sinks (float [n_q] or null): exp(sinks[h]) joins the softmax's denominator (no key, no value, not scaled, no bias).
+// keep_first > 0 (with a window): keys at positions below keep_first stay visible behind the window, at their own positions.
+// n_v (a divisor of n_kv): the value pages hold n_v heads, and key head g reads value head g / (n_kv / n_v).
 template <typename T>
 __global__ void __launch_bounds__(ATT_WAVES * WAVE)
 paged_attention_generic(const T* __restrict__ q, int q_stride, T* __restrict__ out,
@@ -20,7 +22,7 @@ paged_attention_generic(const T* __restrict__ q, int q_stride, T* __restrict__ o
                         const int* __restrict__ positions, const int* __restrict__ entry_of_token,
                         const int* __restrict__ block_table, int table_stride,
                         int n_q, int n_kv, int d, int page_size, int window, float scale, int dv, int chunk,
-                        const float* __restrict__ slopes, const float* __restrict__ sinks) {
+                        const float* __restrict__ slopes, const float* __restrict__ sinks, int keep_first, int n_v) {
   __shared__ float q_s[ATT_MAX_D];
   __shared__ float acc_s[ATT_WAVES][ATT_MAX_D];
   __shared__ float m_s[ATT_WAVES], l_s[ATT_WAVES];
@@ -32,9 +34,13 @@ paged_attention_generic(const T* __restrict__ q, int q_stride, T* __restrict__ o
   const int pos = positions[t];
   const int* table = block_table + (size_t)entry * table_stride;
   const int kvh = h / (n_q / n_kv);
+  const int vh = kvh / (n_kv / n_v);
   int lo = (window >= 0 && pos > window) ? pos - window : 0;
   if (chunk > 0) lo = max(lo, pos / chunk * chunk);
-  const int n_keys = pos - lo + 1;
+  // The keys a query sees, numbered 0..n_keys-1: the kept first ones (positions 0..first-1), then lo..pos.
+  const int first = keep_first > 0 ? min(keep_first, lo) : 0;
+  const int n_keys = first + pos - lo + 1;
+#define KEY_OF(index) ((index) < first ? (index) : lo + (index) - first)
   const float slope = slopes ? slopes[h] : 0.f;
 
   for (int i = threadIdx.x; i < d; i += blockDim.x) q_s[i] = ld(q + (size_t)t * q_stride + (size_t)h * d + i);
@@ -44,14 +50,14 @@ paged_attention_generic(const T* __restrict__ q, int q_stride, T* __restrict__ o
   float m = -INFINITY, l = 0.f;
 
   for (int base = wave * WAVE; base < n_keys; base += ATT_WAVES * WAVE) {
-    const int j = lo + base + lane;
+    const int j = KEY_OF(base + lane);
     const bool valid = base + lane < n_keys;
     int row = 0, vbase = 0;   // key row, and start of this key's column in the value page
     float s = -INFINITY;
     if (valid) {
       const int page = table[j / page_size];
       row = (page * n_kv + kvh) * page_size + (j % page_size);
-      vbase = (page * n_kv + kvh) * page_size * dv + (j % page_size);
+      vbase = (page * n_v + vh) * page_size * dv + (j % page_size);
       const T* kr = k_pages + (size_t)row * d;
       float dot = 0.f;
       if (sizeof(T) == 4 && d % 4 == 0) {
@@ -80,11 +86,12 @@ paged_attention_generic(const T* __restrict__ q, int q_stride, T* __restrict__ o
       __builtin_amdgcn_wave_barrier();
       int jj = 0;
       while (jj < count) {
-        const int j = lo + base + jj;
+        const int j = KEY_OF(base + jj);
         const int off = j % page_size;
-        const int run = min(count - jj, page_size - off);
+        int run = min(count - jj, page_size - off);
+        if (base + jj < first) run = min(run, first - (base + jj));      // a run ends where the kept keys end
         const float* page_v = reinterpret_cast<const float*>(v_pages) +
-                              ((size_t)table[j / page_size] * n_kv + kvh) * dv * page_size + off;
+                              ((size_t)table[j / page_size] * n_v + vh) * dv * page_size + off;
         if (off % 4 == 0 && run >= 4) {
           for (int q4 = 0; q4 + 4 <= run; q4 += 4) {
             const float p0 = p_s[wave][jj + q4], p1 = p_s[wave][jj + q4 + 1], p2 = p_s[wave][jj + q4 + 2],
@@ -144,6 +151,7 @@ paged_attention_generic(const T* __restrict__ q, int q_stride, T* __restrict__ o
     for (int w = 0; w < ATT_WAVES; ++w) v += acc_s[w][i] * weights[w];
     st(out + (size_t)t * n_q * dv + (size_t)h * dv + i, v / denom);
   }
+#undef KEY_OF
 }
 
 extern "C" int ta_paged_attention_generic(const void* q, int q_stride, void* out, const void* k_pages,
@@ -151,20 +159,21 @@ extern "C" int ta_paged_attention_generic(const void* q, int q_stride, void* out
                                           const void* block_table, int table_stride, int n_tokens, int n_q,
                                           int n_kv, int d, int page_size, int window, float scale, int dtype,
                                           int dv, int chunk, const void* slopes, const void* sinks,
-                                          hipStream_t stream) {
+                                          int keep_first, int n_v, hipStream_t stream) {
   if (n_tokens <= 0) return 0;
   if (dv <= 0) dv = d;
-  if (d > ATT_MAX_D || dv > ATT_MAX_D || d <= 0 || n_kv <= 0 || n_q % n_kv) return -1;
+  if (n_v <= 0) n_v = n_kv;
+  if (d > ATT_MAX_D || dv > ATT_MAX_D || d <= 0 || n_kv <= 0 || n_q % n_kv || n_kv % n_v || keep_first < 0) return -1;
   dim3 grid(n_tokens, n_q);
   if (dtype == DT_F32)
     paged_attention_generic<float><<<grid, ATT_WAVES * WAVE, 0, stream>>>((const float*)q, q_stride, (float*)out,
         (const float*)k_pages, (const float*)v_pages, (const int*)positions, (const int*)entry_of_token,
         (const int*)block_table, table_stride, n_q, n_kv, d, page_size, window, scale, dv, chunk,
-        (const float*)slopes, (const float*)sinks);
+        (const float*)slopes, (const float*)sinks, keep_first, n_v);
   else
     paged_attention_generic<bf16_t><<<grid, ATT_WAVES * WAVE, 0, stream>>>((const bf16_t*)q, q_stride, (bf16_t*)out,
         (const bf16_t*)k_pages, (const bf16_t*)v_pages, (const int*)positions, (const int*)entry_of_token,
         (const int*)block_table, table_stride, n_q, n_kv, d, page_size, window, scale, dv, chunk,
-        (const float*)slopes, (const float*)sinks);
+        (const float*)slopes, (const float*)sinks, keep_first, n_v);
   return LAUNCH_STATUS();
 }

@@ -1,0 +1,152 @@
+// Routed feed-forwards and the per-layer token input: the choice of experts from float router logits, the gated
+// activation of the chosen experts with their weights folded in, and the gate of the token input.
+#include "common.h"
+
+__device__ __forceinline__ float rt_gelu_tanh(float z) {
+  return 0.5f * z * (1.0f + tanhf(0.7978845608028654f * (z + 0.044715f * z * z * z)));
+}
+
+// logits: float [n_tokens, n_experts].  For every token the `top` largest logits (the lower index of equals) in falling
+// order: chosen [n_tokens, top] and weights [n_tokens, top] = softmax over those logits alone.  A wave a token.
+__global__ void __launch_bounds__(256)
+route_top_kernel(const float* __restrict__ logits, int n_tokens, int n_experts, int top, int* __restrict__ chosen,
+                 float* __restrict__ weights) {
+  const int lane = threadIdx.x & (WAVE - 1);
+  const int t = blockIdx.x * (blockDim.x / WAVE) + threadIdx.x / WAVE;
+  if (t >= n_tokens) return;
+  const float* row = logits + (size_t)t * n_experts;
+  float top_value = 0.f, total = 0.f, mine = 0.f;
+  int last = -1;
+  float last_value = INFINITY;
+  for (int k = 0; k < top; ++k) {
+    // The largest logit that comes behind the one picked last in the order (value falling, index rising).
+    float best = -INFINITY;
+    int best_at = n_experts;
+    for (int e = lane; e < n_experts; e += WAVE) {
+      const float v = row[e];
+      const bool behind = v < last_value || (v == last_value && e > last);
+      if (behind && (v > best || (v == best && e < best_at))) { best = v; best_at = e; }
+    }
+#pragma unroll
+    for (int off = WAVE / 2; off > 0; off >>= 1) {
+      const float other = __shfl_xor(best, off, WAVE);
+      const int other_at = __shfl_xor(best_at, off, WAVE);
+      if (other > best || (other == best && other_at < best_at)) { best = other; best_at = other_at; }
+    }
+    if (k == 0) top_value = best;
+    const float e = expf(best - top_value);
+    total += e;
+    if (lane == k) mine = e;                        // lane k keeps pick k's term
+    if (lane == 0) chosen[(size_t)t * top + k] = best_at;
+    last = best_at;
+    last_value = best;
+  }
+  // Every lane holds the same total, lane k pick k's term (the launcher takes top <= 64).
+  if (lane < top) weights[(size_t)t * top + lane] = mine / total;
+}
+
+// gate_up: [n_tokens, n_experts * 2 * inner + 2 * shared], expert e's gate rows then its up rows, the shared expert
+// last.  out: [n_tokens, columns] with columns >= n_experts * inner + shared: out[t, e * inner + i] =
+// w * silu(gate) * up for an expert the token chose with weight w, 0 for the others; the shared expert's columns
+// with weight 1; columns beyond are 0.
+template <typename T>
+__global__ void expert_gate_kernel(const T* __restrict__ gate_up, const int* __restrict__ chosen,
+                                   const float* __restrict__ weights, int top, int n_experts, int inner, int shared,
+                                   int columns, T* __restrict__ out, size_t total) {
+  const int in_stride = n_experts * 2 * inner + 2 * shared;
+  for (size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x; idx < total; idx += (size_t)gridDim.x * blockDim.x) {
+    const size_t t = idx / columns;
+    const int c = (int)(idx - t * columns);
+    const T* row = gate_up + t * in_stride;
+    float value = 0.f;
+    if (c < n_experts * inner) {
+      const int e = c / inner, i = c - e * inner;
+      float w = 0.f;
+      for (int k = 0; k < top; ++k)
+        if (chosen[t * top + k] == e) w += weights[t * top + k];
+      if (w != 0.f) {
+        const float g = ld(row + (size_t)e * 2 * inner + i), u = ld(row + (size_t)e * 2 * inner + inner + i);
+        value = w * (g / (1.0f + expf(-g)) * u);
+      }
+    } else if (c < n_experts * inner + shared) {
+      const int i = c - n_experts * inner;
+      const float g = ld(row + (size_t)n_experts * 2 * inner + i), u = ld(row + (size_t)n_experts * 2 * inner + shared + i);
+      value = g / (1.0f + expf(-g)) * u;
+    }
+    st(out + idx, value);
+  }
+}
+
+// out[t, j] = gelu_tanh(gate[t, j]) * table[token_ids[t], offset + j] for j < dim, 0 for dim <= j < columns.
+// gate, out: [n_tokens, columns]; table: [vocab, table_width].
+template <typename T>
+__global__ void side_gate_kernel(const T* __restrict__ gate, const T* __restrict__ table, int table_width,
+                                 const int* __restrict__ token_ids, int offset, int dim, int columns,
+                                 T* __restrict__ out, size_t total) {
+  for (size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x; idx < total; idx += (size_t)gridDim.x * blockDim.x) {
+    const size_t t = idx / columns;
+    const int j = (int)(idx - t * columns);
+    float value = 0.f;
+    if (j < dim) value = rt_gelu_tanh(ld(gate + idx)) * ld(table + (size_t)token_ids[t] * table_width + offset + j);
+    st(out + idx, value);
+  }
+}
+
+// out[t, j] = gelu_tanh(in[t, j]) * in[t, inner + j].
+template <typename T>
+__global__ void gelu_gate_kernel(const T* __restrict__ in, T* __restrict__ out, int inner, size_t total) {
+  for (size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x; idx < total; idx += (size_t)gridDim.x * blockDim.x) {
+    const size_t t = idx / inner;
+    const int j = (int)(idx - t * inner);
+    st(out + idx, rt_gelu_tanh(ld(in + t * 2 * inner + j)) * ld(in + t * 2 * inner + inner + j));
+  }
+}
+
+static inline int rt_blocks(size_t total) { return (int)((total + 255) / 256 < 65535 ? (total + 255) / 256 : 65535); }
+
+extern "C" int ta_route_top(const void* logits, int n_tokens, int n_experts, int top, void* chosen, void* weights,
+                            hipStream_t stream) {
+  if (n_tokens <= 0) return 0;
+  if (top <= 0 || top > n_experts || top > WAVE) return -1;
+  route_top_kernel<<<(n_tokens + 3) / 4, 256, 0, stream>>>((const float*)logits, n_tokens, n_experts, top, (int*)chosen,
+                                                           (float*)weights);
+  return LAUNCH_STATUS();
+}
+
+extern "C" int ta_expert_gate(const void* gate_up, const void* chosen, const void* weights, int n_tokens, int top,
+                              int n_experts, int inner, int shared, int columns, void* out, int dtype, hipStream_t stream) {
+  const size_t total = (size_t)n_tokens * columns;
+  if (total == 0) return 0;
+  if (columns < n_experts * inner + shared) return -1;
+  if (dtype == DT_F32)
+    expert_gate_kernel<float><<<rt_blocks(total), 256, 0, stream>>>((const float*)gate_up, (const int*)chosen,
+        (const float*)weights, top, n_experts, inner, shared, columns, (float*)out, total);
+  else
+    expert_gate_kernel<bf16_t><<<rt_blocks(total), 256, 0, stream>>>((const bf16_t*)gate_up, (const int*)chosen,
+        (const float*)weights, top, n_experts, inner, shared, columns, (bf16_t*)out, total);
+  return LAUNCH_STATUS();
+}
+
+extern "C" int ta_side_gate(const void* gate, const void* table, int table_width, const void* token_ids, int offset, int dim,
+                            int columns, int n_tokens, void* out, int dtype, hipStream_t stream) {
+  const size_t total = (size_t)n_tokens * columns;
+  if (total == 0) return 0;
+  if (dim > columns || offset < 0 || offset + dim > table_width) return -1;
+  if (dtype == DT_F32)
+    side_gate_kernel<float><<<rt_blocks(total), 256, 0, stream>>>((const float*)gate, (const float*)table, table_width,
+        (const int*)token_ids, offset, dim, columns, (float*)out, total);
+  else
+    side_gate_kernel<bf16_t><<<rt_blocks(total), 256, 0, stream>>>((const bf16_t*)gate, (const bf16_t*)table, table_width,
+        (const int*)token_ids, offset, dim, columns, (bf16_t*)out, total);
+  return LAUNCH_STATUS();
+}
+
+extern "C" int ta_gelu_gate(const void* in, void* out, int n_tokens, int inner, int dtype, hipStream_t stream) {
+  const size_t total = (size_t)n_tokens * inner;
+  if (total == 0) return 0;
+  if (dtype == DT_F32)
+    gelu_gate_kernel<float><<<rt_blocks(total), 256, 0, stream>>>((const float*)in, (float*)out, inner, total);
+  else
+    gelu_gate_kernel<bf16_t><<<rt_blocks(total), 256, 0, stream>>>((const bf16_t*)in, (bf16_t*)out, inner, total);
+  return LAUNCH_STATUS();
+}

@@ -154,7 +154,8 @@ class Ops:
                      "ta_splitk_reduce", "ta_splitk_add_rmsnorm", "ta_argmax", "ta_argmax_next_step", "ta_sample",
                      "ta_sample_workspace_words", "ta_library_gemm_bf16", "ta_compute_units", "ta_read_stream",
                      "ta_embedding_streams", "ta_streams_step", "ta_token_shift", "ta_mlstm_scan", "ta_mlstm_chunked", "ta_head_norm_gate",
-                     "ta_capped_gate"):
+                     "ta_capped_gate", "ta_norm_add_rmsnorm", "ta_norm_rotate_store", "ta_differential_heads",
+                     "ta_sigmoid_head_gate", "ta_route_top", "ta_expert_gate", "ta_side_gate", "ta_gelu_gate"):
             getattr(self.lib, name).restype = ctypes.c_int
         self.lib.ta_library_gemm_bf16.argtypes = [ctypes.c_void_p] * 4 + [ctypes.c_int] * 5 + [
             ctypes.c_void_p, ctypes.c_size_t, ctypes.c_int, ctypes.c_void_p]
@@ -267,14 +268,150 @@ class Ops:
                                             _code(out.dtype), self._stream()), "add_rmsnorm")
         return out
 
+    def norm_add_rmsnorm(self, residual: torch.Tensor, delta: torch.Tensor | None, post_weight: torch.Tensor | None,
+                         post_eps: float, weight: torch.Tensor | None, eps: float, out: torch.Tensor,
+                         rows: torch.Tensor | None = None, store_residual: bool = True) -> torch.Tensor:
+        """The norm behind a sub-layer, the residual add and the norm before the next one in one kernel:
+        x = residual + delta / sqrt(mean(delta^2) + post_eps) * post_weight (delta as it is without `post_weight`,
+        nothing without `delta`), stored back into `residual` unless `rows` selects a subset or `store_residual` is
+        off; out = x / sqrt(mean(x^2) + eps) * weight, or x itself without `weight`.
+
+        residual float32 [T, H]; delta [T, H] float32 or bfloat16; weights float32 [H]; rows int32 or None; out
+        [rows, H] in delta's dtype or float32."""
+        _dev(residual, delta, post_weight, weight, out, rows)
+        hidden = residual.shape[1]
+        n_rows = residual.shape[0] if rows is None else rows.numel()
+        _need(residual.dtype == torch.float32 and residual.is_contiguous(), "the residual stream is float32")
+        _need(tuple(out.shape) == (n_rows, hidden) and out.is_contiguous(), "norm output shape")
+        for vector in (post_weight, weight):
+            _need(vector is None or (vector.dtype == torch.float32 and vector.numel() == hidden), "norm weights are float32 [H]")
+        if delta is not None:
+            _need(delta.shape == residual.shape and delta.is_contiguous(), "delta must match the residual's shape")
+            _need(out.dtype in (delta.dtype, torch.float32), "out has delta's dtype or float32")
+        if rows is not None:
+            _need(rows.dtype == torch.int32 and not store_residual, "a row subset (int32) never stores the residual")
+        delta_code = _code(delta.dtype) if delta is not None else _code(out.dtype)
+        self._check(self.lib.ta_norm_add_rmsnorm(_ptr(residual), _ptr(delta), _ptr(post_weight), ctypes.c_float(post_eps),
+                                                 _ptr(weight), ctypes.c_float(eps), _ptr(out), _ptr(rows), n_rows, hidden,
+                                                 int(store_residual and delta is not None), delta_code, _code(out.dtype),
+                                                 self._stream()), "norm_add_rmsnorm")
+        return out
+
+    def norm_rotate_store(self, qkv: torch.Tensor, bias: torch.Tensor | None, positions: torch.Tensor,
+                          rates: torch.Tensor | None, dims: int, slots: torch.Tensor | None,
+                          k_pages: torch.Tensor | None, v_pages: torch.Tensor | None, n_q: int, n_k: int, n_v: int,
+                          d: int, dv: int, q_norm: torch.Tensor | None = None, k_norm: torch.Tensor | None = None,
+                          eps: float = 0.0) -> None:
+        """In place on rows of `qkv` ([T, >= (n_q + n_k) d + n_v dv]: query heads, key heads, value heads): bias; an RMS
+        norm with weight `q_norm` (float32 [n_q d]) over all query elements at once, `k_norm` likewise over the keys;
+        rotation of coordinates i and i + dims / 2 (i < dims / 2) of every query and key head by position * rates[i]
+        (float32 angles, accurate sine and cosine; the coordinates from `dims` on pass); keys and values written at
+        `slots` into key pages [n_pages, n_k, page_size, d] and value pages [n_pages, n_v, dv, page_size]."""
+        _dev(qkv, bias, positions, rates, slots, k_pages, v_pages, q_norm, k_norm)
+        n_tokens, width = qkv.shape
+        used = (n_q + n_k) * d + n_v * dv
+        _need(width >= used and qkv.stride(1) == 1, "qkv is narrower than its heads")
+        _need(positions.dtype == torch.int32 and positions.numel() == n_tokens, "positions must be int32 [T]")
+        _need(dims % 2 == 0 and 0 <= dims <= d and dims <= 256, "the rotation covers an even number of a head's coordinates")
+        if dims:
+            _need(rates is not None and rates.dtype == torch.float32 and rates.numel() == dims // 2, "rates are float32 [dims / 2]")
+        if bias is not None:
+            _need(bias.dtype == torch.float32 and bias.numel() >= used, "bias must be float32 over the heads")
+        _need(q_norm is None or (q_norm.dtype == torch.float32 and q_norm.numel() == n_q * d), "q_norm is float32 [n_q d]")
+        _need(k_norm is None or (k_norm.dtype == torch.float32 and k_norm.numel() == n_k * d), "k_norm is float32 [n_k d]")
+        page_size = 1
+        if slots is not None:
+            _need(slots.dtype == torch.int32 and slots.numel() == n_tokens, "slots must be int32 [T]")
+            _need(k_pages is not None and v_pages is not None, "slots without pages")
+            _need(k_pages.dtype == qkv.dtype and v_pages.dtype == qkv.dtype, "pages must have the dtype of qkv")
+            page_size = self._page_size(k_pages, v_pages, n_k, d, dv, n_v)
+        self._check(self.lib.ta_norm_rotate_store(
+            _ptr(qkv), qkv.stride(0), _ptr(bias), _ptr(positions), _ptr(rates if dims else None), dims, _ptr(slots),
+            _ptr(k_pages), _ptr(v_pages), n_tokens, n_q, n_k, n_v, d, dv, page_size, _ptr(q_norm), _ptr(k_norm),
+            ctypes.c_float(eps), _code(qkv.dtype), self._stream()), "norm_rotate_store")
+
+    def differential_heads(self, mixed: torch.Tensor, lam: torch.Tensor, eps: float, out_scale: float, n_heads: int,
+                           group: int, dv: int, out: torch.Tensor) -> torch.Tensor:
+        """mixed [T, 2 n_heads dv], laid out (kv head, map, head within the group of `group`, dv); out [T, n_heads dv]:
+        o = map 1 - lam[0] * map 2 per head, o / sqrt(mean(o^2) + eps) * out_scale.  lam float32 [1]."""
+        _dev(mixed, lam, out)
+        n_tokens = mixed.shape[0]
+        _need(mixed.is_contiguous() and tuple(mixed.shape) == (n_tokens, 2 * n_heads * dv), "the maps' outputs are [T, 2 H dv]")
+        _need(out.is_contiguous() and tuple(out.shape) == (n_tokens, n_heads * dv) and out.dtype == mixed.dtype, "out is [T, H dv]")
+        _need(lam.dtype == torch.float32 and lam.numel() == 1 and 0 < dv <= 256 and n_heads % group == 0, "lam is float32 [1]")
+        self._check(self.lib.ta_differential_heads(_ptr(mixed), _ptr(lam), ctypes.c_float(eps), ctypes.c_float(out_scale),
+                                                   n_tokens, n_heads, group, dv, _ptr(out), _code(out.dtype), self._stream()),
+                    "differential_heads")
+        return out
+
+    def sigmoid_head_gate(self, mixed: torch.Tensor, rows: torch.Tensor, offset: int, n_heads: int, dv: int) -> torch.Tensor:
+        """mixed[t, h, :] *= sigmoid(rows[t, offset + h]) in place; mixed [T, n_heads dv], rows [T, >= offset + n_heads]."""
+        _dev(mixed, rows)
+        n_tokens = mixed.shape[0]
+        _need(mixed.is_contiguous() and tuple(mixed.shape) == (n_tokens, n_heads * dv), "mixed is [T, H dv]")
+        _need(rows.shape[0] == n_tokens and rows.stride(1) == 1 and rows.shape[1] >= offset + n_heads and rows.dtype == mixed.dtype,
+              "the gates' rows do not fit")
+        self._check(self.lib.ta_sigmoid_head_gate(_ptr(mixed), _ptr(rows), rows.stride(0), offset, n_tokens, n_heads, dv,
+                                                  _code(mixed.dtype), self._stream()), "sigmoid_head_gate")
+        return mixed
+
+    def route_top(self, logits: torch.Tensor, chosen: torch.Tensor, weights: torch.Tensor) -> None:
+        """For every row of float32 `logits` [T, E]: the indices of its `top` largest (chosen int32 [T, top], falling
+        order, the lower index of equals first) and the softmax over those alone (weights float32 [T, top])."""
+        _dev(logits, chosen, weights)
+        n_tokens, n_experts = logits.shape
+        top = chosen.shape[1]
+        _need(logits.dtype == torch.float32 and logits.is_contiguous(), "router logits are float32")
+        _need(chosen.dtype == torch.int32 and weights.dtype == torch.float32 and chosen.is_contiguous() and weights.is_contiguous()
+              and tuple(chosen.shape) == (n_tokens, top) == tuple(weights.shape), "chosen int32 and weights float32 [T, top]")
+        _need(0 < top <= min(n_experts, 64), "between one and 64 experts a token, no more than there are")
+        self._check(self.lib.ta_route_top(_ptr(logits), n_tokens, n_experts, top, _ptr(chosen), _ptr(weights), self._stream()),
+                    "route_top")
+
+    def expert_gate(self, gate_up: torch.Tensor, chosen: torch.Tensor, weights: torch.Tensor, n_experts: int, inner: int,
+                    shared: int, out: torch.Tensor) -> torch.Tensor:
+        """gate_up [T, n_experts 2 inner + 2 shared] (every expert's gate rows, then its up rows; the shared expert
+        last) -> out [T, >= n_experts inner + shared]: weight * silu(gate) * up in the columns of the experts a token
+        chose, silu(gate) * up in the shared expert's, zero everywhere else."""
+        _dev(gate_up, chosen, weights, out)
+        n_tokens = gate_up.shape[0]
+        _need(gate_up.is_contiguous() and gate_up.shape[1] == n_experts * 2 * inner + 2 * shared, "gate_up width")
+        _need(out.is_contiguous() and out.shape[0] == n_tokens and out.shape[1] >= n_experts * inner + shared
+              and out.dtype == gate_up.dtype, "out is [T, >= E inner + shared]")
+        _need(chosen.dtype == torch.int32 and weights.dtype == torch.float32 and chosen.shape == weights.shape
+              and chosen.shape[0] == n_tokens and chosen.is_contiguous() and weights.is_contiguous(), "chosen and weights [T, top]")
+        self._check(self.lib.ta_expert_gate(_ptr(gate_up), _ptr(chosen), _ptr(weights), n_tokens, chosen.shape[1], n_experts,
+                                            inner, shared, out.shape[1], _ptr(out), _code(out.dtype), self._stream()),
+                    "expert_gate")
+        return out
+
+    def side_gate(self, gate: torch.Tensor, table: torch.Tensor, token_ids: torch.Tensor, offset: int, dim: int,
+                  out: torch.Tensor) -> torch.Tensor:
+        """out[t, j] = gelu_tanh(gate[t, j]) * table[token_ids[t], offset + j] for j < dim, zero in further columns."""
+        _dev(gate, table, token_ids, out)
+        n_tokens, columns = gate.shape
+        _need(gate.is_contiguous() and out.is_contiguous() and out.shape == gate.shape and out.dtype == gate.dtype == table.dtype,
+              "gate and out are [T, columns] of the table's dtype")
+        _need(table.dim() == 2 and table.is_contiguous() and 0 <= offset and offset + dim <= table.shape[1] and dim <= columns,
+              "the table's slice")
+        _need(token_ids.dtype == torch.int32 and token_ids.numel() == n_tokens, "token ids are int32 [T]")
+        self._check(self.lib.ta_side_gate(_ptr(gate), _ptr(table), table.shape[1], _ptr(token_ids), offset, dim, columns,
+                                          n_tokens, _ptr(out), _code(out.dtype), self._stream()), "side_gate")
+        return out
+
     # ------------------------------------------------------------- gated activation
     def silu_gate(self, gate_up: torch.Tensor, out: torch.Tensor, act: tuple | None = None) -> torch.Tensor:
         """out = silu(gate_up[:, :I]) * gate_up[:, I:].  gate_up [T, 2I]; out [T, I].  With `act` = (alpha, limit,
-        shift): g' = min(g, limit), u' = clamp(u, -limit, limit), out = g' * sigmoid(alpha g') * (u' + shift)."""
+        shift): g' = min(g, limit), u' = clamp(u, -limit, limit), out = g' * sigmoid(alpha g') * (u' + shift); with
+        `act` = "gelu_tanh": out = 0.5 g (1 + tanh(sqrt(2/pi) (g + 0.044715 g^3))) * u."""
         _dev(gate_up, out)
         n_tokens, two_inner = gate_up.shape
         _need(two_inner % 2 == 0 and tuple(out.shape) == (n_tokens, two_inner // 2) and out.dtype == gate_up.dtype,
               "silu_gate shapes do not fit")
+        if act == "gelu_tanh":
+            self._check(self.lib.ta_gelu_gate(_ptr(gate_up), _ptr(out), n_tokens, two_inner // 2, _code(out.dtype),
+                                              self._stream()), "gelu_gate")
+            return out
         if act is not None:
             alpha, limit, shift = act
             self._check(self.lib.ta_capped_gate(_ptr(gate_up), _ptr(out), n_tokens, two_inner // 2, ctypes.c_float(alpha),
@@ -319,12 +456,12 @@ class Ops:
 
     @staticmethod
     def _page_size(k_pages: torch.Tensor, v_pages: torch.Tensor, n_kv: int, head_dim: int,
-                   value_dim: int | None = None) -> int:
+                   value_dim: int | None = None, value_heads: int | None = None) -> int:
         value_dim = head_dim if value_dim is None else value_dim
         _need(k_pages.dim() == 4 and k_pages.shape[1] == n_kv and k_pages.shape[3] == head_dim,
               "key pages must be [n_pages, n_kv, page_size, d]")
         page_size = k_pages.shape[2]
-        _need(tuple(v_pages.shape) == (k_pages.shape[0], n_kv, value_dim, page_size),
+        _need(tuple(v_pages.shape) == (k_pages.shape[0], n_kv if value_heads is None else value_heads, value_dim, page_size),
               "value pages must be [n_pages, n_kv, dv, page_size]")
         _need(k_pages.numel() < 2 ** 31 and v_pages.numel() < 2 ** 31, "a layer's pages must hold fewer than 2^31 elements")
         return page_size
@@ -335,8 +472,13 @@ class Ops:
                         block_table: torch.Tensor, n_q: int, n_kv: int, head_dim: int,
                         window: int | None, scale: float, max_position: int | None = None,
                         batch=None, value_dim: int | None = None, chunk: int | None = None,
-                        slopes: torch.Tensor | None = None, sinks: torch.Tensor | None = None) -> torch.Tensor:
+                        slopes: torch.Tensor | None = None, sinks: torch.Tensor | None = None,
+                        keep_first: int = 0, value_heads: int | None = None) -> torch.Tensor:
         """Causal attention of every token over the pages of its request.
+
+        `keep_first` n (with a window): keys at positions below n stay visible behind the window.  `value_heads`
+        (a divisor of n_kv): the value pages hold so many heads, and key head g reads value head
+        g / (n_kv / value_heads).  Both run the generic kernel.
 
         Beyond the plain form: `value_dim` (value heads of dv elements; out is [T, n_q dv]), `chunk` (only keys
         of the query's own run of so many positions, counted from position 0), `slopes` (float32 [n_q]: head h's
@@ -358,10 +500,13 @@ class Ops:
             _need(extra is None or (extra.dtype == torch.float32 and extra.numel() == n_q), "slopes and sinks are float32 [n_q]")
         _need(chunk is None or chunk > 0, "a chunk has at least one position")
         plain = value_dim == head_dim and chunk is None and slopes is None and sinks is None
+        value_heads = n_kv if value_heads is None else int(value_heads)
+        keep_first = int(keep_first) if window is not None else 0
+        _need(value_heads > 0 and n_kv % value_heads == 0 and keep_first >= 0, "value heads divide the key heads")
         _need(qkv.shape[1] >= n_q * head_dim, "qkv is narrower than the query heads")
         _need(tuple(out.shape) == (n_tokens, n_q * value_dim) and out.dtype == qkv.dtype, "attention output shape")
         _need(k_pages.dtype == qkv.dtype and v_pages.dtype == qkv.dtype, "pages must have the dtype of qkv")
-        page_size = self._page_size(k_pages, v_pages, n_kv, head_dim, value_dim)
+        page_size = self._page_size(k_pages, v_pages, n_kv, head_dim, value_dim, value_heads)
         _need(positions.dtype == torch.int32 and positions.numel() == n_tokens, "positions must be int32 [T]")
         _need(entry_of_token.dtype == torch.int32 and entry_of_token.numel() == n_tokens, "entry_of_token must be int32 [T]")
         _need(block_table.dtype == torch.int32 and block_table.dim() == 2, "block_table must be int32 [E, P]")
@@ -372,7 +517,7 @@ class Ops:
         # The matrix-core kernels take chunks, slopes and sinks as they are; value heads of another size than the key
         # heads go to the generic kernel.
         if (value_dim == head_dim and qkv.dtype == torch.bfloat16 and head_dim in self.DECODE_HEAD_DIMS and page_size % 16 == 0
-                and qkv.shape[1] % 8 == 0 and self.use_fast_attention):
+                and qkv.shape[1] % 8 == 0 and self.use_fast_attention and keep_first == 0 and value_heads == n_kv):
             args = (qkv, out, k_pages, v_pages, positions, entry_of_token, block_table, n_q, n_kv, head_dim,
                     page_size, window, scale, max_position)
             extras = {} if plain else dict(chunk=chunk, slopes=slopes, sinks=sinks)
@@ -407,7 +552,8 @@ class Ops:
             _ptr(qkv), qkv.shape[1], _ptr(out), _ptr(k_pages), _ptr(v_pages), _ptr(positions),
             _ptr(entry_of_token), _ptr(block_table), block_table.shape[1], n_tokens, n_q, n_kv, head_dim,
             page_size, -1 if window is None else int(window), ctypes.c_float(scale), _code(qkv.dtype),
-            value_dim, 0 if chunk is None else int(chunk), _ptr(slopes), _ptr(sinks), self._stream()), "paged_attention")
+            value_dim, 0 if chunk is None else int(chunk), _ptr(slopes), _ptr(sinks), keep_first, value_heads,
+            self._stream()), "paged_attention")
         return out
 
     DECODE_HEAD_DIMS = (16, 32, 48, 64, 80, 96, 112, 128, 160, 192, 224, 256)
