@@ -165,7 +165,7 @@ def routed_ff(h: torch.Tensor, w: dict, mlp: dict) -> torch.Tensor:
             out[t] += p * gated_ff(h[t:t + 1], one, silu)[0]
     if mlp.get("shared"):
         out = out + gated_ff(h, {name: w[f"shared.{name}"] for name in ("gate", "up", "down")}, silu)
-    assert experts == sum(1 for name in w if name.startswith("e") and name.endswith(".gate"))
+    assert logits.shape[-1] == experts
     return out
 
 
@@ -220,3 +220,13 @@ def forward(cfg: dict, tensors: dict, tokens, return_layers: bool = False):
         after.append(x)
     logits = weighted_norm(x, tensors["final.norm"], eps) @ tensors["head"].T
     return (logits, after) if return_layers else logits
+
+
+def greedy_generate(cfg: dict, tensors: dict, prompt, n_new: int) -> list[int]:
+    """The first maximum of the last position's logits, appended and run again from the start, `n_new` times."""
+    ids, out = list(prompt), []
+    for _ in range(n_new):
+        logits = forward(cfg, tensors, ids)[-1]
+        out.append(int(torch.argmax(logits)))
+        ids.append(out[-1])
+    return out

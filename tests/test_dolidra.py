@@ -1,0 +1,548 @@
+"""Dolidra through the framework against the plain implementation of tests/plain/dolidra_plain.py.
+
+Every test runs on three backends: the engine on the CPU with the plain torch ops standing in for the kernel
+library (the host side: tables, slots, cache units, batching), and the engine on the GPU in float32 and in bfloat16
+(the HIP kernels).  The models are the tiny ones of dolidra_configs.py with sharpened weights.
+"""
+import numpy as np
+import pytest
+import torch
+
+import trace_tools as tt
+from dolidra_configs import DOLIDRA, write_model
+from plain import dolidra_plain as plain
+from tiny_configs import random_ids
+
+BACKENDS = [pytest.param("cpu", id="cpu"),
+            pytest.param("gpu-float32", marks=pytest.mark.gpu, id="gpu-float32"),
+            pytest.param("gpu-bfloat16", marks=pytest.mark.gpu, id="gpu-bfloat16")]
+# float32: sums in another order, against logits of order 1.  bfloat16 rounds the activations between the kernels and
+# the sharpened weights carry that further than a trained model's would: there the bound is on each row's root mean
+# square error against the row's own spread (a key too many, a window one off or a lost kept key moves a row by its
+# whole spread; float32 pins the same kernels' indexing to five digits).
+TOL = {"cpu": 2e-5, "gpu-float32": 5e-5, "gpu-bfloat16": 0.12}
+
+
+@pytest.fixture(scope="module")
+def folders(tmp_path_factory):
+    root = tmp_path_factory.mktemp("dolidra")
+    return {name: write_model(raw, seed, str(root / name)) for name, (raw, seed) in DOLIDRA.items()}
+
+
+@pytest.fixture(scope="module")
+def oracle(folders):
+    cache = {}
+
+    def get(name, ids):
+        key = (name, tuple(ids))
+        if key not in cache:
+            cfg, tensors = plain.load_folder(folders[name])
+            cache[key] = plain.forward(cfg, tensors, list(ids)).to(torch.float32)
+        return cache[key]
+    return get
+
+
+def make_engine(folder, backend, **kw):
+    from tokenizer_amd.engine import Engine, load_model
+    if backend == "cpu":
+        from kernel_refs import PlainOps
+        return Engine(load_model(folder, "float32", "cpu", ops=PlainOps()), **kw)
+    return Engine(load_model(folder, backend.split("-")[1]), **kw)
+
+
+def close(got, want, backend, what=""):
+    got = got.float().cpu()
+    if backend == "gpu-bfloat16":
+        spread = (want - want.mean(dim=-1, keepdim=True)).pow(2).mean(dim=-1).sqrt()
+        off = (got - want).pow(2).mean(dim=-1).sqrt() / spread
+        assert float(off.max()) <= 4 * TOL[backend] and int((off > TOL[backend]).sum()) <= max(1, off.numel() // 50), \
+            f"{what}: rows are off by up to {float(off.max())} of their spread, {int((off > TOL[backend]).sum())} over the bound"
+        return
+    err = float((got - want).abs().max())
+    bound = TOL[backend] * max(float(want.abs().max()), 1.0)
+    assert err <= bound, f"{what}: max abs error {err} against a bound of {bound}"
+
+
+def requests_for(name, lengths=(1, 2, 3, 21, 50, 97, 64, 33)):
+    vocab = DOLIDRA[name][0]["vocab"]
+    return {f"r{i}": random_ids(vocab, n, 40 + i) for i, n in enumerate(lengths)}
+
+
+def check_trace(folders, oracle, name, backend, steps, reqs, **kw):
+    eng = make_engine(folders[name], backend, max_tokens=tt.peak_tokens(steps), max_requests=4, **kw)
+    eng.pools.poison()          # pages that no request wrote read as NaN
+    got = tt.run_in_process(eng, steps)
+    for rid, ids in reqs.items():
+        close(got[rid], oracle(name, ids), backend, rid)
+    eng.cache.check_invariants()
+    assert not eng.cache.requests
+    return eng
+
+
+SMALL = ["A", "B", "C", "D"]
+
+
+@pytest.mark.parametrize("backend", BACKENDS)
+@pytest.mark.parametrize("name", SMALL)
+def test_whole_prompts_and_the_first_tokens(folders, oracle, name, backend):
+    reqs = requests_for(name)
+    check_trace(folders, oracle, name, backend, tt.whole(reqs), reqs)
+
+
+@pytest.mark.parametrize("backend", BACKENDS)
+@pytest.mark.parametrize("name", SMALL)
+def test_prefill_then_token_by_token(folders, oracle, name, backend):
+    # The tail of 50 carries every window of the models (1 to 48 positions) and the kept first positions over decoded
+    # tokens, and passes page borders of 16.
+    reqs = requests_for(name, (60, 97, 64, 51))
+    check_trace(folders, oracle, name, backend, tt.decode_tail(reqs, 50), reqs)
+
+
+@pytest.mark.parametrize("backend", BACKENDS)
+@pytest.mark.parametrize("name", SMALL)
+@pytest.mark.parametrize("seed", [3, 4])
+def test_portions_down_to_two_tokens(folders, oracle, name, backend, seed):
+    reqs = requests_for(name, (97, 50, 64, 7))
+    steps = tt.portions(reqs, seed)
+    assert any(len(s["entries"][0]["tokens"]) == 2 for s in steps)
+    check_trace(folders, oracle, name, backend, steps, reqs)
+
+
+@pytest.mark.parametrize("backend", BACKENDS)
+@pytest.mark.parametrize("name", SMALL)
+@pytest.mark.parametrize("seed", [6, 7])
+def test_mixed_batches_with_pages_and_slots_used_again(folders, oracle, name, backend, seed):
+    reqs = requests_for(name, (33, 97, 21, 64, 50, 80, 12, 45, 3, 70))
+    steps = tt.mixed(reqs, seed, max_live=4, tail=14)
+    assert max(len(s["entries"]) for s in steps) >= 3
+    eng = check_trace(folders, oracle, name, backend, steps, reqs)
+    assert eng.cache.max_requests == 4          # ten requests went through four slots
+
+
+@pytest.mark.parametrize("backend", BACKENDS)
+@pytest.mark.parametrize("page_size", [16, 48])
+def test_other_page_sizes_and_batches_against_each_request_alone(folders, oracle, backend, page_size):
+    from tokenizer_amd.engine import StepEntry
+    name = "A"
+    reqs = requests_for(name, (70, 9, 31))
+    eng = make_engine(folders[name], backend, num_pages=24, page_size=page_size, max_requests=3)
+    eng.pools.poison()
+    for rid in reqs:
+        eng.add_request(rid)
+    heads = {rid: len(ids) - 5 for rid, ids in reqs.items()}
+    got = {rid: [] for rid in reqs}
+    logits = eng.step([StepEntry(rid, ids[:heads[rid]], list(range(heads[rid]))) for rid, ids in reqs.items()]).float().cpu()
+    row = 0
+    for rid in reqs:
+        got[rid].append(logits[row:row + heads[rid]])
+        row += heads[rid]
+    for k in range(5):
+        logits = eng.step([StepEntry(rid, [ids[heads[rid] + k]], [0]) for rid, ids in reqs.items()]).float().cpu()
+        for row, rid in enumerate(reqs):
+            got[rid].append(logits[row:row + 1])
+    for rid, ids in reqs.items():
+        close(torch.cat(got[rid]), oracle(name, ids), backend, rid)
+
+
+@pytest.mark.parametrize("backend", BACKENDS)
+@pytest.mark.parametrize("name", ["A", "C"])
+def test_long_decoding(folders, oracle, name, backend):
+    ids = random_ids(DOLIDRA[name][0]["vocab"], 230, 77)
+    reqs = {"long": ids}
+    check_trace(folders, oracle, name, backend, tt.decode_tail(reqs, tail=227), reqs)
+
+
+@pytest.mark.parametrize("backend", BACKENDS)
+def test_greedy_generation_through_the_entry_point_and_the_scheduler(folders, backend):
+    from tokenizer_amd.engine import GenerateParams, Scheduler, SchedulerConfig, generate
+    name = "A"
+    cfg, tensors = plain.load_folder(folders[name])
+    prompts = [random_ids(cfg["vocab"], n, 90 + n) for n in (11, 30, 4)]
+    want = [plain.greedy_generate(cfg, tensors, p, 9) for p in prompts]
+    eng = make_engine(folders[name], backend, num_pages=16, max_requests=4)
+    eng.pools.poison()
+    alone = [generate(eng, p, GenerateParams.greedy(9)).tokens for p in prompts]
+    sched = Scheduler(eng, SchedulerConfig(num_blocks=16, max_batch_size=4))
+    rids = [sched.add_request(p, GenerateParams.greedy(9)) for p in prompts]
+    results = sched.run()
+    together = [results[rid].tokens for rid in rids]
+    assert alone == together
+    if backend != "gpu-bfloat16":           # (bfloat16 may pick another of two near-equal logits)
+        assert alone == want
+    else:
+        assert sum(a == w for a, w in zip(sum(alone, []), sum(want, []))) >= 20
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("cut", ["whole", "tail", "portions", "mixed"])
+def test_hundreds_of_tokens_with_long_windows(folders, oracle, dtype, cut):
+    """Contexts of up to 900 tokens under windows of 260, 300 and 520 with kept first positions hundreds of tokens
+    back: keys far away, window edges deep in a prompt and among decoded tokens."""
+    name = "E"
+    reqs = {f"r{i}": random_ids(DOLIDRA[name][0]["vocab"], n, 70 + i) for i, n in enumerate((900, 333, 610, 545))}
+    steps = {"whole": lambda: tt.whole(reqs), "tail": lambda: tt.decode_tail(reqs, 48),
+             "portions": lambda: tt.portions(reqs, 9), "mixed": lambda: tt.mixed(reqs, 12, max_live=3, tail=30)}[cut]()
+    check_trace(folders, oracle, name, "gpu-" + dtype, steps, reqs)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_the_replay_program_on_a_model_folder(folders, oracle, tmp_path, dtype):
+    """bin/trace_run as a child process: the class is chosen by config.json, the pool is made for the trace's peak,
+    four slots serve ten requests."""
+    name = "D"
+    reqs = requests_for(name, (33, 97, 21, 64, 50, 80, 12, 45, 3, 70))
+    steps = tt.mixed(reqs, 11, max_live=4, tail=14)
+    got = tt.run_program(folders[name], dtype, steps, str(tmp_path / "out"), tt.peak_tokens(steps), DOLIDRA[name][0]["vocab"])
+    for rid, ids in reqs.items():
+        close(got[rid], oracle(name, ids), "gpu-" + dtype, rid)
+
+
+# ------------------------------------------------------------------ configuration, schedule, cache
+def test_the_schedule_gives_every_pass_of_a_looped_layer_its_own_cache():
+    from tokenizer_amd.config import DolidraConfig
+    from tokenizer_amd.models.dolidra import dolidra_spec
+    from tokenizer_amd.parts import cache_needs
+    spec = dolidra_spec(DolidraConfig.from_dict(DOLIDRA["A"][0]))
+    assert [entry.layer for entry in spec.schedule] == plain.run_order(DOLIDRA["A"][0]) == [0, 1, 2, 1, 2, 3]
+    units = [entry.cache_unit() for entry in spec.schedule]
+    assert len(set(units)) == len(units) and units == [0, 1, 2, 4, 5, 3]
+    needs = cache_needs(spec)
+    assert len(needs) == 6 and needs[4] == needs[1] and needs[5] == needs[2]
+    # Differential layers keep a key head per map and one value head per kv head.
+    assert (needs[0].n_kv_heads, needs[0].v_heads, needs[0].head_dim, needs[0].v_dim) == (4, 2, 16, 24)
+    assert (needs[1].kind, needs[1].window, needs[1].keep_first) == ("window", 11, 5)
+    assert needs[3].kind == "full"
+
+
+def test_a_config_with_a_missing_or_misfitting_key_is_refused():
+    from tokenizer_amd.config import ConfigError, DolidraConfig
+    raw = DOLIDRA["A"][0]
+    for path, value in ((("layers", 0, "mixer", "rot", "dims"), 7), (("layers", 1, "mlp", "router", "top"), 9),
+                        (("loop", "stop"), 9), (("layers", 0, "mixer", "kv_heads"), 3), (("layers", 2, "type"), "mlstm")):
+        import copy
+        broken = copy.deepcopy(raw)
+        at = broken
+        for key in path[:-1]:
+            at = at[key]
+        at[path[-1]] = value
+        with pytest.raises(ConfigError):
+            DolidraConfig.from_dict(broken)
+
+
+def test_pages_behind_a_window_go_back_but_those_of_the_kept_positions_stay():
+    from tokenizer_amd.cache import CacheManager
+    from tokenizer_amd.parts.spec import CacheNeed
+    needs = [CacheNeed("window", 2, 16, window=39, keep_first=20), CacheNeed("window", 2, 16, window=39)]
+    manager = CacheManager(needs, num_pages=32, page_size=16, max_requests=2)
+    manager.add_request("a")
+    assert manager.reserve("a", 200)
+    manager.advance("a", 200)
+    kept, plain_window = manager.table("a", 0), manager.table("a", 1)
+    # Position 200 reads back to 160: pages 0..9 are behind it; the first twenty positions lie in pages 0 and 1.
+    assert [p >= 0 for p in kept] == [True, True] + [False] * 8 + [True] * 3
+    assert [p >= 0 for p in plain_window] == [False] * 10 + [True] * 3
+    manager.release("a")
+    manager.check_invariants()
+    assert manager.groups[0].allocator.available() == 32 and manager.groups[1].allocator.available() == 32
+
+
+def test_the_rates_of_the_rotation_with_scaled_long_waves():
+    from tokenizer_amd.parts.position import scaled_rates
+    for rot in ({"dims": 8, "base": 10000.0, "scaling": {"factor": 4.0, "low": 1.0, "high": 4.0, "original": 64}},
+                {"dims": 48, "base": 250000.0, "scaling": {"factor": 8.0, "low": 1.0, "high": 2.0, "original": 100}},
+                {"dims": 6, "base": 100.0}):
+        want = plain.rotation_rates(rot)
+        got = scaled_rates(rot["base"], rot["dims"], rot.get("scaling")).double()
+        assert float(((got - want) / want).abs().max()) < 1e-7
+    # All three ranges occur in the first one: kept, mixed, slowed.
+    ratios = (plain.rotation_rates({"dims": 8, "base": 10000.0, "scaling": {"factor": 4.0, "low": 1.0, "high": 4.0, "original": 64}})
+              / plain.rotation_rates({"dims": 8, "base": 10000.0}))
+    assert ratios[0] == 1.0 and 0.25 < ratios[1] < 1.0 and ratios[2] == 0.25 and ratios[3] == 0.25
+
+
+# ------------------------------------------------------------------ mechanisms alone
+def ops_for(backend):
+    if backend == "cpu":
+        from kernel_refs import PlainOps
+        return PlainOps(), torch.device("cpu"), torch.float32
+    from tokenizer_amd.kernels import get_ops
+    return get_ops(), torch.device("cuda:0"), (torch.float32 if backend.endswith("float32") else torch.bfloat16)
+
+
+def rounded(x, dtype):
+    """Random float64 data as the compute dtype holds it."""
+    return x.to(dtype).to(torch.float64)
+
+
+def tolerance(dtype, exact=2e-5, rough=3e-2):
+    return rough if dtype == torch.bfloat16 else exact
+
+
+class Batch:
+    """A batch description made by hand: entries of (first position, rows)."""
+
+    def __init__(self, entries, device):
+        i32 = lambda values: torch.tensor(values, dtype=torch.int32, device=device)
+        self.cu_q = i32(np.cumsum([0] + [n for _, n in entries]).tolist())
+        self.first_position = i32([p for p, _ in entries])
+        self.entry_of_token = i32([e for e, (_, n) in enumerate(entries) for _ in range(n)])
+        self.positions = i32([p + k for p, n in entries for k in range(n)])
+        self.n_tokens = int(self.cu_q[-1])
+        tiles = [[e, at] for e, (_, n) in enumerate(entries) if n != 1 for at in range(0, n, 16)]
+        self.q_tiles = i32(tiles).reshape(-1, 2)
+        rows = np.cumsum([0] + [n for _, n in entries])
+        self.decode_rows = i32([int(rows[e]) for e, (_, n) in enumerate(entries) if n == 1])
+        self.max_position = max(p + n - 1 for p, n in entries)
+
+
+@pytest.mark.parametrize("backend", BACKENDS)
+@pytest.mark.parametrize("width", [64, 52, 200, 4352])
+def test_the_norm_behind_a_sub_layer_with_the_add_and_the_next_norm(backend, width):
+    ops, device, dtype = ops_for(backend)
+    gen = torch.Generator().manual_seed(width)
+    rand = lambda *shape: torch.randn(*shape, generator=gen, dtype=torch.float64)
+    tokens, eps_b, eps = 5, 3e-5, 1e-6
+    x = (3.0 * rand(tokens, width)).float().double()
+    y = rounded(7.0 * rand(tokens, width), dtype)
+    behind, before = (rand(width) * 0.3 + 1).float().double(), (rand(width) * 0.3 + 1).float().double()
+    new = x + plain.weighted_norm(y, behind, eps_b)
+    want = plain.weighted_norm(new, before, eps)
+    dev = lambda t, kind=torch.float32: t.to(kind).to(device)
+    held = dev(x)
+    got = torch.empty((tokens, width), dtype=dtype, device=device)
+    ops.norm_add_rmsnorm(held, dev(y, dtype), dev(behind), eps_b, dev(before), eps, got)
+    tol = tolerance(dtype)
+    assert float((got.double().cpu() - want).abs().max()) <= tol * float(want.abs().max())
+    assert float((held.double().cpu() - new).abs().max()) <= 1e-5 * float(new.abs().max())
+    # Without a norm before the next sub-layer the sum itself comes out; a subset of rows stores nothing.
+    held = dev(x)
+    rows = torch.tensor([3, 0], dtype=torch.int32, device=device)
+    got = torch.empty((2, width), dtype=dtype, device=device)
+    ops.norm_add_rmsnorm(held, dev(y, dtype), dev(behind), eps_b, None, 0.0, got, rows, store_residual=False)
+    assert float((got.double().cpu() - new[[3, 0]]).abs().max()) <= tol * float(new.abs().max())
+    assert torch.equal(held.cpu(), x.float())
+    # Nothing to add: the norm of the stream as it is.
+    got = torch.empty((tokens, width), dtype=dtype, device=device)
+    ops.norm_add_rmsnorm(held, None, None, 0.0, dev(before), eps, got)
+    assert float((got.double().cpu() - plain.weighted_norm(x, before, eps)).abs().max()) <= tol * float(want.abs().max())
+
+
+@pytest.mark.parametrize("backend", BACKENDS)
+@pytest.mark.parametrize("n_q,n_k,n_v,d,dv,dims,normed,bias", [(4, 2, 2, 16, 24, 8, False, True), (6, 3, 3, 12, 14, 12, True, False),
+                                                              (8, 4, 2, 32, 32, 32, False, True), (2, 1, 1, 64, 64, 16, True, False),
+                                                              (3, 3, 3, 10, 6, 0, True, True)])
+def test_bias_norm_over_the_whole_projection_partial_rotation_and_the_store(backend, n_q, n_k, n_v, d, dv, dims, normed, bias):
+    ops, device, dtype = ops_for(backend)
+    gen = torch.Generator().manual_seed(n_q * d + dims)
+    rand = lambda *shape: torch.randn(*shape, generator=gen, dtype=torch.float64)
+    tokens, page_size, eps, extra = 9, 16, 1e-5, 5
+    used = (n_q + n_k) * d + n_v * dv
+    rows = rounded(rand(tokens, used + extra), dtype)
+    b = rand(used + extra).float().double() if bias else None
+    positions = torch.tensor([0, 1, 2, 700, 701, 31, 15, 16, 4095])
+    rot = {"dims": dims, "base": 250000.0, "scaling": {"factor": 4.0, "low": 1.0, "high": 4.0, "original": 2048}}
+    rates = plain.rotation_rates(rot) if dims else torch.zeros(0, dtype=torch.float64)
+    wq, wk = (rand(n_q * d) * 0.3 + 1).float().double(), (rand(n_k * d) * 0.3 + 1).float().double()
+    x = rows[:, :used] + (b[:used] if bias else 0)
+    q, k, v = x[:, :n_q * d], x[:, n_q * d:(n_q + n_k) * d], x[:, (n_q + n_k) * d:]
+    if normed:
+        q, k = plain.weighted_norm(q, wq, eps), plain.weighted_norm(k, wk, eps)
+    q = plain.rotate(q.reshape(tokens, n_q, d), positions, rates).reshape(tokens, -1)
+    k = plain.rotate(k.reshape(tokens, n_k, d), positions, rates).reshape(tokens, -1)
+    dev = lambda t, kind=torch.float32: None if t is None else t.to(kind).to(device)
+    held = dev(rows, dtype)
+    k_pages = torch.full((6, n_k, page_size, d), float("nan"), dtype=dtype, device=device)
+    v_pages = torch.full((6, n_v, dv, page_size), float("nan"), dtype=dtype, device=device)
+    slots = torch.tensor([5 * 16 + 3, 0, 17, -1, 2 * 16 + 15, 3 * 16, 4 * 16 + 7, 1, 95], dtype=torch.int32, device=device)
+    ops.norm_rotate_store(held, dev(b), dev(positions, torch.int32), dev(rates) if dims else None, dims, slots, k_pages, v_pages,
+                          n_q, n_k, n_v, d, dv, dev(wq) if normed else None, dev(wk) if normed else None, eps)
+    # (The angle is a float32 product, as the design has it: at position 4,095 it is off by up to 3e-4 of a radian
+    # from the exact one, which is what the bound leaves room for.)
+    tol = tolerance(dtype, 4e-4) * max(1.0, float(x.abs().max()))
+    got = held.double().cpu()
+    assert float((got[:, :n_q * d] - q).abs().max()) <= tol and float((got[:, n_q * d:(n_q + n_k) * d] - k).abs().max()) <= tol
+    assert float((got[:, (n_q + n_k) * d:used] - v).abs().max()) <= tol
+    assert torch.equal(got[:, used:], rows[:, used:])                     # what lies behind the heads is left alone
+    for t, slot in enumerate(slots.tolist()):
+        if slot < 0:
+            continue
+        page, off = divmod(slot, page_size)
+        assert torch.equal(k_pages[page, :, off, :].reshape(-1).cpu(), held[t, n_q * d:(n_q + n_k) * d].cpu())
+        assert torch.equal(v_pages[page, :, :, off].reshape(-1).cpu(), held[t, (n_q + n_k) * d:used].cpu())
+    written = {divmod(s, page_size) for s in slots.tolist() if s >= 0}
+    for page in range(6):
+        for off in range(page_size):
+            if (page, off) not in written:
+                assert bool(torch.isnan(k_pages[page, :, off, :].float()).all())
+
+
+def run_attention(ops, device, dtype, q, k, v, cuts, window, keep_first, share, scale, page_size=16):
+    """One sequence through the cache in steps of `cuts` tokens (a second, short sequence rides along in every step so
+    that the batch is never one entry): the keys go through the store kernel without rotation, the queries through the
+    attention.  q [n, n_q, d], k [n, n_k, d], v [n, n_k / share, dv] -> [n, n_q, dv]."""
+    n, n_q, d = q.shape
+    n_k, n_v, dv = k.shape[1], v.shape[1], v.shape[2]
+    n_pages = -(-n // page_size) + 2
+    k_pages = torch.full((n_pages, n_k, page_size, d), float("nan"), dtype=dtype, device=device)
+    v_pages = torch.full((n_pages, n_v, dv, page_size), float("nan"), dtype=dtype, device=device)
+    order = list(reversed(range(n_pages - 1)))                   # the sequence's pages in falling order; the last is the rider's
+    table = torch.tensor([order, [n_pages - 1] + [-1] * (n_pages - 2)], dtype=torch.int32, device=device)
+    rows = torch.cat([q.reshape(n, -1), k.reshape(n, -1), v.reshape(n, -1)], dim=1).to(dtype).to(device)
+    out, at, rider = [], 0, 0
+    for size in cuts:
+        batch = Batch([(at, size), (rider, 1)], device)
+        step = torch.cat([rows[at:at + size], rows[rider:rider + 1]]).contiguous()
+        slots = [order[p // page_size] * page_size + p % page_size for p in range(at, at + size)] + [(n_pages - 1) * page_size + rider]
+        ops.norm_rotate_store(step, None, batch.positions, None, 0, torch.tensor(slots, dtype=torch.int32, device=device),
+                              k_pages, v_pages, n_q, n_k, n_v, d, dv)
+        mixed = torch.zeros((size + 1, n_q * dv), dtype=dtype, device=device)
+        ops.paged_attention(step, mixed, k_pages, v_pages, batch.positions, batch.entry_of_token, table, n_q, n_k, d,
+                            window, scale, max_position=batch.max_position, batch=batch, value_dim=dv,
+                            keep_first=keep_first, value_heads=n_v)
+        out.append(mixed[:size].double().cpu())
+        at, rider = at + size, (rider + 1) % page_size
+    return torch.cat(out).reshape(n, n_q, dv)
+
+
+CUTS = {"prompt": lambda n: [n], "portions": lambda n: [37, 2, 16, 1, 1, 29] + [n - 86],
+        "decoded": lambda n: [n - 70] + [1] * 70}
+
+
+@pytest.mark.parametrize("backend", BACKENDS)
+@pytest.mark.parametrize("cut", list(CUTS))
+@pytest.mark.parametrize("n_q,n_k,share,d,dv,size,keep", [(4, 2, 1, 16, 24, 40, 20), (4, 4, 2, 16, 8, 23, 0), (6, 2, 1, 32, 32, 16, 17),
+                                                         (8, 2, 2, 64, 64, 33, 0), (2, 1, 1, 48, 48, 64, 5), (3, 3, 1, 12, 14, 1, 3)])
+def test_one_key_made_to_stand_out_at_every_edge(backend, cut, n_q, n_k, share, d, dv, size, keep):
+    """Every query is made to score one chosen key far above all others: the key just inside its window, just outside
+    it, the last kept first position, the one behind it, the keys on either side of a page border, a key far back and
+    itself, in turn.  A mask that is one position off then changes the output by all of it."""
+    ops, device, dtype = ops_for(backend)
+    n = 150
+    gen = torch.Generator().manual_seed(size * 100 + keep)
+    rand = lambda *shape: torch.randn(*shape, generator=gen, dtype=torch.float64)
+    k = rand(n, n_k, d)
+    k = k / k.norm(dim=-1, keepdim=True)
+    v = rand(n, n_k // share, dv)
+    q = 0.3 * rand(n, n_q, d)
+    group = n_q // n_k
+    for i in range(n):
+        choices = [i - size + 1, i - size, keep - 1, keep, i - i % 16, i - i % 16 - 1, 1, i]
+        j = choices[i % len(choices)]
+        if 0 <= j <= i:
+            for h in range(n_q):
+                q[i, h] += 12.0 * k[j, h // group]
+    q, k, v = rounded(q, dtype), rounded(k, dtype), rounded(v, dtype)
+    got = run_attention(ops, device, dtype, q, k, v, CUTS[cut](n), size - 1, keep, share, 1.0)
+    seen = plain.visible(n, size, keep)
+    want = torch.stack([plain.masked_softmax_attention(q[:, h], k[:, h // group], v[:, h // group // share], 1.0, seen)
+                        for h in range(n_q)], dim=1)
+    assert float((got - want).abs().max()) <= tolerance(dtype, 2e-5, 4e-2) * float(want.abs().max())
+    # The chosen keys do carry the outputs: without the kept positions, or with a window one longer, rows move by far more.
+    for other in (plain.visible(n, size + 1, keep), plain.visible(n, size, max(keep - 1, 0)) if keep else plain.visible(n, size - 1 or 2, 0)):
+        moved = torch.stack([plain.masked_softmax_attention(q[:, h], k[:, h // group], v[:, h // group // share], 1.0, other)
+                             for h in range(n_q)], dim=1)
+        assert float((moved - want).abs().max()) > 0.5
+
+
+@pytest.mark.parametrize("backend", BACKENDS)
+@pytest.mark.parametrize("heads,kv_heads,d,dv,diff", [(4, 2, 16, 24, 0.3), (3, 3, 12, 14, 0.8), (8, 1, 16, 256, 0.5), (2, 1, 32, 100, 0.0)])
+def test_the_difference_of_two_maps_per_head(backend, heads, kv_heads, d, dv, diff):
+    ops, device, dtype = ops_for(backend)
+    gen = torch.Generator().manual_seed(heads * dv)
+    rand = lambda *shape: torch.randn(*shape, generator=gen, dtype=torch.float64)
+    tokens, eps, group = 7, 1e-5, heads // kv_heads
+    maps = rounded(rand(tokens, heads, 2, dv), dtype)                     # by head, as the design lays them out
+    lam = torch.tensor([0.37 + diff], dtype=torch.float64)
+    want = (plain.unit_rms(maps[:, :, 0] - lam * maps[:, :, 1], eps) * (1 - diff)).reshape(tokens, -1)
+    # The kernels' order: (kv head, map, head within the group).
+    laid = maps.reshape(tokens, kv_heads, group, 2, dv).transpose(2, 3).reshape(tokens, -1)
+    out = torch.empty((tokens, heads * dv), dtype=dtype, device=device)
+    ops.differential_heads(laid.to(dtype).to(device), lam.float().to(device), eps, 1 - diff, heads, group, dv, out)
+    assert float((out.double().cpu() - want).abs().max()) <= tolerance(dtype) * max(1.0, float(want.abs().max()))
+
+
+@pytest.mark.parametrize("backend", BACKENDS)
+def test_the_gate_per_head(backend):
+    ops, device, dtype = ops_for(backend)
+    gen = torch.Generator().manual_seed(9)
+    tokens, heads, dv, offset = 6, 5, 14, 11
+    mixed = rounded(torch.randn(tokens, heads, dv, generator=gen, dtype=torch.float64), dtype)
+    rows = rounded(3 * torch.randn(tokens, offset + heads + 2, generator=gen, dtype=torch.float64), dtype)
+    want = mixed * torch.sigmoid(rows[:, offset:offset + heads])[:, :, None]
+    got = mixed.reshape(tokens, -1).to(dtype).to(device).contiguous()
+    ops.sigmoid_head_gate(got, rows.to(dtype).to(device), offset, heads, dv)
+    assert float((got.double().cpu().reshape(tokens, heads, dv) - want).abs().max()) <= tolerance(dtype) * float(want.abs().max())
+
+
+@pytest.mark.parametrize("backend", BACKENDS)
+@pytest.mark.parametrize("experts,top,inner,shared,width", [(5, 2, 24, 40, 64), (3, 1, 20, 0, 48), (12, 3, 10, 6, 52), (70, 8, 16, 8, 32)])
+def test_routing_and_the_experts(backend, experts, top, inner, shared, width):
+    ops, device, dtype = ops_for(backend)
+    gen = torch.Generator().manual_seed(experts * top)
+    rand = lambda *shape: torch.randn(*shape, generator=gen, dtype=torch.float64)
+    tokens = 19
+    h = rounded(rand(tokens, width), dtype)
+    w = {"router": rounded(rand(experts, width) * 0.5, dtype)}
+    names = [f"e{j}" for j in range(experts)] + (["shared"] if shared else [])
+    for name in names:
+        size = shared if name == "shared" else inner
+        w.update({f"{name}.gate": rounded(rand(size, width) * 0.3, dtype), f"{name}.up": rounded(rand(size, width) * 0.3, dtype),
+                  f"{name}.down": rounded(rand(width, size) * 0.3, dtype)})
+    mlp = {"router": {"experts": experts, "top": top}, "shared": {"ff": shared} if shared else None}
+    want = plain.routed_ff(h, w, mlp)
+    dev = lambda t: t.to(dtype).to(device).contiguous()
+    logits = ops.linear(dev(h), dev(w["router"]), out_dtype=torch.float32)
+    chosen = torch.empty((tokens, top), dtype=torch.int32, device=device)
+    weights = torch.empty((tokens, top), dtype=torch.float32, device=device)
+    ops.route_top(logits, chosen, weights)
+    exact = h @ w["router"].T
+    picked, order = torch.topk(exact, top, dim=-1)
+    assert torch.equal(chosen.cpu().long(), order)
+    assert float((weights.double().cpu() - torch.softmax(picked, dim=-1)).abs().max()) <= 1e-5
+    gate_up = ops.linear(dev(h), dev(torch.cat([w[f"{name}.{part}"] for name in names for part in ("gate", "up")])))
+    fill = (-(experts * inner + shared)) % 8
+    act = torch.full((tokens, experts * inner + shared + fill), float("nan"), dtype=dtype, device=device)
+    ops.expert_gate(gate_up, chosen, weights, experts, inner, shared, act)
+    down = torch.cat([w[f"{name}.down"] for name in names] + [torch.zeros(width, fill, dtype=torch.float64)], dim=1)
+    got = ops.linear(act, dev(down))
+    assert float((got.double().cpu() - want).abs().max()) <= tolerance(dtype, 3e-5, 4e-2) * float(want.abs().max())
+    # An expert no token chose contributes exact zeros.
+    columns = act.double().cpu()[:, :experts * inner].reshape(tokens, experts, inner)
+    for t in range(tokens):
+        for e in range(experts):
+            assert bool((columns[t, e] == 0).all()) == (e not in order[t].tolist())
+
+
+@pytest.mark.parametrize("backend", BACKENDS)
+@pytest.mark.parametrize("dim,columns", [(6, 8), (16, 16), (3, 3)])
+def test_the_token_input_and_the_tanh_gelu_gate(backend, dim, columns):
+    ops, device, dtype = ops_for(backend)
+    if dtype != torch.bfloat16:
+        columns = dim
+    gen = torch.Generator().manual_seed(dim)
+    rand = lambda *shape: torch.randn(*shape, generator=gen, dtype=torch.float64)
+    tokens, vocab, layers, layer, width, eps = 9, 31, 4, 2, 40, 1e-5
+    table = rounded(rand(vocab, layers * dim), dtype)
+    ids = torch.randint(0, vocab, (tokens,), generator=gen)
+    x = rounded(2 * rand(tokens, width), dtype)
+    w = {"gate": rounded(rand(dim, width) * 0.4, dtype), "proj": rounded(rand(width, dim), dtype), "norm": rand(width).float().double()}
+    want = plain.token_side_input(x, ids, table, w, layer, dim, eps)
+    dev = lambda t, kind=None: t.to(kind or dtype).to(device).contiguous()
+    pad = lambda m, rows, cols: torch.cat([torch.cat([m, torch.zeros(m.shape[0], cols - m.shape[1], dtype=m.dtype)], dim=1),
+                                           torch.zeros(rows - m.shape[0], cols, dtype=m.dtype)], dim=0)
+    gate = ops.linear(dev(x), dev(pad(w["gate"], columns, width)))
+    gated = torch.full((tokens, columns), float("nan"), dtype=dtype, device=device)
+    ops.side_gate(gate, dev(table), dev(ids, torch.int32), layer * dim, dim, gated)
+    assert bool((gated[:, dim:] == 0).all())
+    y = ops.linear(gated, dev(pad(w["proj"], width, columns)))
+    stream = torch.zeros((tokens, width), dtype=torch.float32, device=device)
+    ops.norm_add_rmsnorm(stream, y, dev(w["norm"], torch.float32), eps, None, 0.0, torch.empty_like(y))
+    assert float((stream.double().cpu() - want).abs().max()) <= tolerance(dtype, 3e-5, 5e-2) * float(want.abs().max())
+    # The dense feed-forward's activation.
+    gate_up = rounded(3 * rand(tokens, 2 * 22), dtype)
+    out = torch.empty((tokens, 22), dtype=dtype, device=device)
+    ops.silu_gate(dev(gate_up), out, act="gelu_tanh")
+    want = plain.gelu_tanh(gate_up[:, :22]) * gate_up[:, 22:]
+    assert float((out.double().cpu() - want).abs().max()) <= tolerance(dtype) * float(want.abs().max())
