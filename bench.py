@@ -18,7 +18,7 @@ share a prefix of 1,024 ids, with the prefix cache) and prints one JSON line for
 
 times the prompt attention kernel alone on a portion of TOKENS tokens after C cached ones.
 
-    python bench.py --design napadra [--size 0.5b|1.5b|7b] [--layers N] [--batch B] [--steps K]
+    python bench.py --design napadra|dolidra [--size 0.5b|1.5b|7b] [--layers N] [--batch B] [--steps K]
 
 times a prefill of 2,048 tokens and decoding at batch B of a Napadra model whose layers have the sizes of the
 Qwen2.5 model named (width, heads, feed-forward and vocabulary; its layers alternate attention, attention on the
@@ -267,17 +267,51 @@ def napadra_config(sizes: dict, layers: int, chunk: int = 4096, streams: int = 4
             "residual_mult": 0.7, "norm": {"eps": 1e-6}, "layers": out}
 
 
+def dolidra_config(sizes: dict, layers: int, window: int = 4096, keep_first: int = 64, experts: int = 8, top: int = 2) -> dict:
+    """A Dolidra configuration with the layer sizes of a Qwen2 one.  Differential layers have half the heads with two
+    maps each, so that queries and keys are as wide as Qwen2's; the windows are longer than the bench's contexts, so
+    that both models' attention reads the same keys; a routed feed-forward has `experts` experts of a quarter of the
+    dense inner width, of which a token uses `top`, and a shared expert of half of it (as many multiply-adds a token
+    as the dense one).  The layers alternate as differential + dense, differential + routed, gated + dense,
+    differential + routed, and the first two run twice."""
+    width, heads, kv_heads = sizes["hidden_size"], sizes["num_attention_heads"], sizes["num_key_value_heads"]
+    d, inner = width // heads, sizes["intermediate_size"]
+    rot = {"base": float(sizes.get("rope_theta", 1e6)), "dims": d,
+           "scaling": {"factor": 4.0, "low": 1.0, "high": 4.0, "original": 8192}}
+    dense = {"kind": "dense", "ff": inner}
+    routed = {"kind": "moe", "expert": {"ff": inner // 4 // 8 * 8}, "router": {"experts": experts, "top": top},
+              "shared": {"ff": inner // 2 // 8 * 8}}
+    out = []
+    for index in range(layers):
+        kind = index % 4
+        if kind == 2:
+            mixer = {"heads": heads, "kv_heads": kv_heads, "dim": d, "vdim": d, "scale": d ** -0.5,
+                     "mask": {"size": window, "keep_first": keep_first}, "rot": {"base": rot["base"], "dims": d // 4}}
+            out.append({"type": "attention_2", "mixer": mixer, "mlp": dense})
+            continue
+        mixer = {"heads": max(1, heads // 2), "kv_heads": max(1, kv_heads // 2), "dim": d, "vdim": d, "scale": d ** -0.5,
+                 "diff": 0.5, "mask": {"size": window}, "rot": rot}
+        out.append({"type": "attention", "mixer": mixer, "mlp": dense if kind == 0 else routed})
+    return {"architecture": "Dolidra", "vocab": sizes["vocab_size"], "width": width, "norm": {"eps": 1e-6},
+            "token_side": {"dim": 16}, "loop": {"start": 0, "stop": min(2, layers), "times": 2}, "layers": out}
+
+
 def run_design(args, sizes: dict) -> dict:
-    """Prefill and decode throughput of Napadra beside Qwen2 at equal layer sizes and count."""
+    """Prefill and decode throughput of the named design beside Qwen2 at equal layer sizes and number of layer runs."""
     import torch
-    from tokenizer_amd.config import NapadraConfig, Qwen2Config
+    from tokenizer_amd.config import DolidraConfig, NapadraConfig, Qwen2Config
     from tokenizer_amd.engine import random_model
     layers = args.layers or 8
     steps = min(args.steps, 256)
-    record = {"design": "napadra", "beside": "qwen2", "size": args.size, "layers": layers, "dtype": args.dtype,
+    record = {"design": args.design, "beside": "qwen2", "size": args.size, "layers": layers, "dtype": args.dtype,
               "prompt_len": PROMPT_LEN, "batch": args.batch, "decode_steps": steps, "data": "synthetic (random weights)"}
-    configs = {"napadra": lambda: NapadraConfig.from_dict(napadra_config(sizes, layers)),
-               "qwen2": lambda: Qwen2Config.from_dict(dict(sizes, num_hidden_layers=layers))}
+    if args.design == "dolidra":
+        # (Two of the layers run twice: `layers` counts the runs, so that both models run as many layers a token.)
+        configs = {"dolidra": lambda: DolidraConfig.from_dict(dolidra_config(sizes, max(2, layers - 2))),
+                   "qwen2": lambda: Qwen2Config.from_dict(dict(sizes, num_hidden_layers=layers))}
+    else:
+        configs = {"napadra": lambda: NapadraConfig.from_dict(napadra_config(sizes, layers)),
+                   "qwen2": lambda: Qwen2Config.from_dict(dict(sizes, num_hidden_layers=layers))}
     for name, make in configs.items():
         if args.only and args.only != name:
             continue
@@ -292,9 +326,9 @@ def run_design(args, sizes: dict) -> dict:
         log(f"{name}: {record[name]}")
         del model
         torch.cuda.empty_cache()
-    if "napadra" in record and "qwen2" in record:
-        record["prefill_ratio"] = round(record["napadra"]["prefill_tokens_per_s"] / record["qwen2"]["prefill_tokens_per_s"], 3)
-        record["decode_ratio"] = round(record["napadra"]["decode_tokens_per_s"] / record["qwen2"]["decode_tokens_per_s"], 3)
+    if args.design in record and "qwen2" in record:
+        record["prefill_ratio"] = round(record[args.design]["prefill_tokens_per_s"] / record["qwen2"]["prefill_tokens_per_s"], 3)
+        record["decode_ratio"] = round(record[args.design]["decode_tokens_per_s"] / record["qwen2"]["decode_tokens_per_s"], 3)
     return record
 
 
@@ -389,9 +423,9 @@ def main() -> int:
     parser.add_argument("--layers", type=int, default=None)
     parser.add_argument("--size", default="0.5b", choices=["0.5b", "1.5b", "7b"],
                         help="layer sizes of the decode benchmark (the default is the one the record is for)")
-    parser.add_argument("--design", default=None, choices=["napadra"],
+    parser.add_argument("--design", default=None, choices=["napadra", "dolidra"],
                         help="time this design beside Qwen2 at equal layer sizes (prefill and decode)")
-    parser.add_argument("--only", default=None, choices=["napadra", "qwen2"], help="with --design: one of the two models")
+    parser.add_argument("--only", default=None, choices=["napadra", "dolidra", "qwen2"], help="with --design: one of the two models")
     parser.add_argument("--peaks", action="store_true", help="measure what the device reaches in HBM reads and bf16 products")
     parser.add_argument("--workload", default=None, choices=["mixed-1.5b", "mixed-0.5b", "prefix-7b"],
                         help="run a serving workload through the scheduler instead of the decode benchmark")

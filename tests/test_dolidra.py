@@ -55,7 +55,10 @@ def close(got, want, backend, what=""):
     if backend == "gpu-bfloat16":
         spread = (want - want.mean(dim=-1, keepdim=True)).pow(2).mean(dim=-1).sqrt()
         off = (got - want).pow(2).mean(dim=-1).sqrt() / spread
-        assert float(off.max()) <= 4 * TOL[backend] and int((off > TOL[backend]).sum()) <= max(1, off.numel() // 50), \
+        # (A router's logits for two experts are now and then nearly equal; bfloat16 rounding then picks the other
+        # expert, and that row, and a few behind it that attend to it, move by a good part of their spread.  Such
+        # rows are few; a wrong mask or a lost key moves every row behind the first window.)
+        assert int((off > TOL[backend]).sum()) <= max(2, off.numel() // 12) and float(off.median()) <= TOL[backend] / 4, \
             f"{what}: rows are off by up to {float(off.max())} of their spread, {int((off > TOL[backend]).sum())} over the bound"
         return
     err = float((got - want).abs().max())
@@ -170,7 +173,11 @@ def test_greedy_generation_through_the_entry_point_and_the_scheduler(folders, ba
     if backend != "gpu-bfloat16":           # (bfloat16 may pick another of two near-equal logits)
         assert alone == want
     else:
-        assert sum(a == w for a, w in zip(sum(alone, []), sum(want, []))) >= 20
+        # Every token it picked is, for the oracle and after the same tokens, the largest logit or within rounding of it.
+        for prompt, picked in zip(prompts, alone):
+            logits = plain.forward(cfg, tensors, prompt + picked)[len(prompt) - 1:-1]
+            for row, token in zip(logits, picked):
+                assert float(row.max() - row[token]) <= 0.15 * float(row.std())
 
 
 @pytest.mark.gpu
@@ -413,7 +420,8 @@ CUTS = {"prompt": lambda n: [n], "portions": lambda n: [37, 2, 16, 1, 1, 29] + [
 @pytest.mark.parametrize("backend", BACKENDS)
 @pytest.mark.parametrize("cut", list(CUTS))
 @pytest.mark.parametrize("n_q,n_k,share,d,dv,size,keep", [(4, 2, 1, 16, 24, 40, 20), (4, 4, 2, 16, 8, 23, 0), (6, 2, 1, 32, 32, 16, 17),
-                                                         (8, 2, 2, 64, 64, 33, 0), (2, 1, 1, 48, 48, 64, 5), (3, 3, 1, 12, 14, 1, 3)])
+                                                         (8, 2, 2, 64, 64, 33, 0), (2, 1, 1, 48, 48, 64, 5), (3, 3, 1, 12, 14, 1, 3),
+                                                         (4, 2, 1, 64, 64, 24, 70), (4, 1, 1, 128, 128, 9, 100), (4, 4, 2, 32, 32, 20, 0)])
 def test_one_key_made_to_stand_out_at_every_edge(backend, cut, n_q, n_k, share, d, dv, size, keep):
     """Every query is made to score one chosen key far above all others: the key just inside its window, just outside
     it, the last kept first position, the one behind it, the keys on either side of a page border, a key far back and

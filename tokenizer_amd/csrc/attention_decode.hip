@@ -27,6 +27,10 @@ __device__ __forceinline__ bf16x8 zero8() {
 // Partials: part_o [n_items, n_q, splits, D] (unnormalised), part_ml [n_items, n_q, splits, 2] (max, sum);
 // with splits == 1 the result goes straight to `out` [n_tokens, n_q * D].
 // AHEAD: a wave asks for its next block of keys while it works on the current one (see below).
+// EXTRA also: keep_first > 0 (with a window): keys at positions below keep_first stay visible behind the window; the
+// last `kept_splits` of the `splits` workgroups of a row walk those keys (positions 0 .. min(keep_first, first key of
+// the window) - 1) and leave their partial state beside the others'.  n_v < n_kv: the value pages hold n_v heads and
+// key head g reads value head g / (n_kv / n_v).
 // EXTRA: chunk > 0: only the keys of the token's own run of `chunk` positions (runs counted from position 0) are seen;
 // slopes (float [n_q] or null): head h's score loses slopes[h] per position between token and key; sinks (float [n_q] or
 // null): exp(sinks[h]) joins the softmax's denominator (it rides in the first split's partial sums).
@@ -38,7 +42,8 @@ decode_attention_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_t* __re
                         const int* __restrict__ entry_of_token, const int* __restrict__ block_table,
                         int table_stride, float* __restrict__ part_o, float* __restrict__ part_ml,
                         int n_q, int n_kv, int page_size, int window, float scale, int split_keys, int splits,
-                        int chunk, const float* __restrict__ slopes, const float* __restrict__ sinks) {
+                        int chunk, const float* __restrict__ slopes, const float* __restrict__ sinks,
+                        int keep_first, int kept_splits, int n_v) {
   constexpr int KS = (D + 31) / 32;   // 32-wide steps over the head size for Q K^T
   constexpr int DB = D / 16;          // 16-row blocks of O^T
   HELD(q, q_stride, out, k_pages, vt_pages, rows, positions, entry_of_token, block_table, table_stride, part_o, part_ml,
@@ -73,8 +78,17 @@ decode_attention_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_t* __re
   int lo = (window >= 0 && pos > window) ? pos - window : 0;
   if (EXTRA && chunk > 0) lo = max(lo, pos / chunk * chunk);
   const float slope = (EXTRA && slopes && col < heads_here) ? slopes[head] : 0.f;
-  const int first = (lo / 32) * 32 + split * split_keys;  // first key of this split (a multiple of 32)
-  const int last = min(pos, first + split_keys - 1);
+  int first = (lo / 32) * 32 + split * split_keys;        // first key of this split (a multiple of 32)
+  int last = min(pos, first + split_keys - 1);
+  int vh = kvh, n_vh = n_kv;                               // the value head this key head reads, of so many
+  if (EXTRA) {
+    if (n_v > 0 && n_v < n_kv) { vh = kvh / (n_kv / n_v); n_vh = n_v; }
+    if (kept_splits > 0 && split >= splits - kept_splits) {       // a split over the kept first keys
+      first = (split - (splits - kept_splits)) * split_keys;
+      last = min(min(keep_first, lo) - 1, first + split_keys - 1);
+      lo = 0;
+    }
+  }
 
   // Q^T fragments: lane holds head `col`, head-size elements ks*32 + 8g .. +7.
   bf16x8 qf[KS];
@@ -141,7 +155,7 @@ decode_attention_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_t* __re
       }
       {
         const int half = g >> 1;
-        const uint32_t at = ((uint32_t)(half ? page1 : page0) * n_kv + kvh) * page_elems + (uint32_t)col * page_size +
+        const uint32_t at = ((uint32_t)(half ? page1 : page0) * n_vh + vh) * page_elems + (uint32_t)col * page_size +
                             ((kb + 16 * half) % page_size) + 8 * (g & 1);
         blk.left = (half ? there1 : there0) ? last - (kb + 8 * g) : -1;
 #pragma unroll
@@ -358,7 +372,8 @@ static int launch_decode(const void* q, int q_stride, void* out, const void* k_p
                          const void* rows, const void* positions, const void* entry_of_token,
                          const void* block_table, int table_stride, void* part_o, void* part_ml, int n_items,
                          int n_q, int n_kv, int page_size, int window, float scale, int split_keys, int splits,
-                         int chunk, const void* slopes, const void* sinks, hipStream_t stream) {
+                         int chunk, const void* slopes, const void* sinks, int keep_first, int kept_splits, int n_v,
+                         hipStream_t stream) {
   const int group = n_q / n_kv;
   dim3 grid(splits, n_kv * ((group + 15) / 16), n_items);
   constexpr int NW = D > 128 ? 2 : 4;   // keeps the merge buffer within 64 KB of LDS
@@ -366,8 +381,8 @@ static int launch_decode(const void* q, int q_stride, void* out, const void* k_p
       (const bf16_t*)q, q_stride, (bf16_t*)out, (const bf16_t*)k_pages, (const bf16_t*)vt_pages, (const int*)rows, \
       (const int*)positions, (const int*)entry_of_token, (const int*)block_table, table_stride, (float*)part_o, \
       (float*)part_ml, n_q, n_kv, page_size, window, scale, split_keys, splits, chunk, (const float*)slopes, \
-      (const float*)sinks)
-  if (chunk > 0 || slopes || sinks) { if (split_keys <= 32 * NW * 8) GO(true, true); else GO(false, true); }
+      (const float*)sinks, keep_first, kept_splits, n_v)
+  if (chunk > 0 || slopes || sinks || kept_splits > 0 || (n_v > 0 && n_v < n_kv)) { if (split_keys <= 32 * NW * 8) GO(true, true); else GO(false, true); }
   else if (split_keys <= 32 * NW * 8) GO(true, false); else GO(false, false);      // up to eight blocks a wave
 #undef GO
   int status = LAUNCH_STATUS();
@@ -398,12 +413,17 @@ extern "C" int ta_decode_attention_bf16(const void* q, int q_stride, void* out, 
                                         const void* entry_of_token, const void* block_table, int table_stride,
                                         void* part_o, void* part_ml, int n_items, int n_q, int n_kv, int d,
                                         int page_size, int window, float scale, int split_keys, int splits,
-                                        int chunk, const void* slopes, const void* sinks, hipStream_t stream) {
+                                        int chunk, const void* slopes, const void* sinks, int keep_first,
+                                        int kept_splits, int n_v, hipStream_t stream) {
   if (n_items <= 0) return 0;
   if (n_kv <= 0 || n_q % n_kv || page_size % 16 || split_keys % 32 || splits < 1) return -1;
+  if (n_v <= 0) n_v = n_kv;
+  if (n_kv % n_v || keep_first < 0 || kept_splits < 0 || kept_splits >= splits || (keep_first > 0) != (kept_splits > 0) ||
+      (long)kept_splits * split_keys < keep_first || (keep_first > 0 && (window < 0 || chunk > 0)))
+    return -1;
 #define CASE(DD) case DD: return launch_decode<DD>(q, q_stride, out, k_pages, vt_pages, rows, positions, entry_of_token, \
     block_table, table_stride, part_o, part_ml, n_items, n_q, n_kv, page_size, window, scale, split_keys, splits, chunk, \
-    slopes, sinks, stream);
+    slopes, sinks, keep_first, kept_splits, n_v, stream);
   switch (d) {
     CASE(16) CASE(32) CASE(48) CASE(64) CASE(80) CASE(96) CASE(112) CASE(128) CASE(160) CASE(192) CASE(224) CASE(256)
     default: return -2;

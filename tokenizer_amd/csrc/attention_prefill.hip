@@ -29,7 +29,11 @@ __device__ __forceinline__ void prefill_block(
     const bf16_t* __restrict__ k_pages, const bf16_t* __restrict__ vt_pages, const int* __restrict__ table,
     int kb, int kvh, int n_kv, int page_size, int col, int g, int heads_here, int my_pos, int my_lo, int lo, int hi,
     float c, const bf16x8 (&qf)[HG][(D + 31) / 32], floatx4 (&acc)[HG][D / 16], float (&m)[HG], float (&l)[HG],
-    const float (&slope)[HG]) {
+    const float (&slope)[HG], int keep_first = 0, int vh = -1, int n_vh = 0) {
+  // EXTRA: keep_first > 0: keys below it stay visible (and their pages readable) behind the window; vh >= 0: the
+  // value pages hold n_vh heads and this key head reads value head vh.
+  if (!EXTRA || vh < 0) { vh = kvh; n_vh = n_kv; }
+  if (!EXTRA) keep_first = 0;
   constexpr int KS = (D + 31) / 32;
   constexpr int DB = D / 16;
   // The block is two halves of 32 keys.  Key base + k of a half is index k of the second product's contraction
@@ -43,7 +47,7 @@ __device__ __forceinline__ void prefill_block(
 #pragma unroll
   for (int u = 0; u < 2; ++u) {
     const int base_key = kb + 32 * u;
-    const bool active = FULL || ((base_key <= hi) && (base_key + 31 >= lo));      // the same for the whole wave
+    const bool active = FULL || ((base_key <= hi) && (base_key + 31 >= lo || base_key < keep_first));   // the same for the whole wave
 #pragma unroll
     for (int t = 0; t < 2; ++t)
 #pragma unroll
@@ -54,7 +58,8 @@ __device__ __forceinline__ void prefill_block(
       // A half's two runs of sixteen keys: one that holds no key of the range (before `lo`: its page may have been
       // given back; after `hi`: it may not exist yet) borrows the other's page, a valid address; what is read
       // there never counts (scores outside the range are masked, such values are set to zero).
-      const bool there0 = FULL || base_key + 15 >= lo, there1 = FULL || base_key + 16 <= hi;
+      const bool there0 = FULL || base_key + 15 >= lo || base_key < keep_first;
+      const bool there1 = FULL || (base_key + 16 <= hi && (base_key + 31 >= lo || base_key + 16 < keep_first));
       const int page0 = scalar_int(table + (there0 ? base_key : base_key + 16) / page_size);
       const int page1 = scalar_int(table + (there1 ? base_key + 16 : base_key) / page_size);
       const uint32_t page_elems = (uint32_t)page_size * D;
@@ -71,7 +76,7 @@ __device__ __forceinline__ void prefill_block(
       }
       {
         const int half = g >> 1;
-        const uint32_t at = ((uint32_t)(half ? page1 : page0) * n_kv + kvh) * page_elems + (uint32_t)col * page_size +
+        const uint32_t at = ((uint32_t)(half ? page1 : page0) * n_vh + vh) * page_elems + (uint32_t)col * page_size +
                             ((base_key + 16 * half) % page_size) + 8 * (g & 1);
         // (Nothing that was loaded is touched before all of the block is asked for: a value that is used makes the
         // wave wait for everything it asked for before.)
@@ -115,7 +120,7 @@ __device__ __forceinline__ void prefill_block(
         if (FULL) {
           s[t * 4 + r] = score;
         } else {
-          s[t * 4 + r] = (key <= my_pos && key >= my_lo) ? score : -INFINITY;
+          s[t * 4 + r] = (key <= my_pos && (key >= my_lo || key < keep_first)) ? score : -INFINITY;
         }
       }
     }
@@ -162,7 +167,8 @@ prefill_attention_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_t* __r
                          const int* __restrict__ tiles, int n_tiles, const int* __restrict__ cu_q,
                          const int* __restrict__ first_position, const int* __restrict__ block_table,
                          int table_stride, int n_q, int n_kv, int page_size, int window, float scale_log2,
-                         int chunk, const float* __restrict__ slopes, const float* __restrict__ sinks, float inv_scale) {
+                         int chunk, const float* __restrict__ slopes, const float* __restrict__ sinks, float inv_scale,
+                         int keep_first, int n_v) {
   constexpr int KS = (D + 31) / 32;
   constexpr int DB = D / 16;
   HELD(q, q_stride, out, k_pages, vt_pages, tiles, n_tiles, cu_q, first_position, block_table, table_stride, n_q, n_kv,
@@ -203,7 +209,10 @@ prefill_attention_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_t* __r
   float slope[HG];
 #pragma unroll
   for (int h = 0; h < HG; ++h) slope[h] = 0.f;
+  int kept = 0, vh = -1, n_vh = 0;      // keys kept visible behind the window; the value head this key head reads, of so many
   if (EXTRA) {
+    kept = window >= 0 ? keep_first : 0;
+    if (n_v > 0 && n_v < n_kv) { vh = kvh / (n_kv / n_v); n_vh = n_v; }
     if (chunk > 0) {          // a token sees the keys of its own run of `chunk` positions only; a tile may lie across two runs
       lo = max(lo, p0 / chunk * chunk);
       lo_all = max(lo_all, hi / chunk * chunk);
@@ -240,16 +249,24 @@ prefill_attention_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_t* __r
   // A wave's blocks come in three runs: those at the window's edge (some keys masked), those that every token
   // of the tile sees whole, and those on the diagonal.  Each run is a loop of its own over one variant of the
   // block: in one loop over both, the accumulators would be copied between the variants' registers every turn.
+  if (EXTRA && kept > 0) {
+    // The kept first keys that lie before the window's first block (those inside the blocks below are let through
+    // by the mask there): every token of the tile sees them.
+    const int kept_end = min(kept, (lo / 64) * 64);
+    for (int k0 = 64 * wave; k0 < kept_end; k0 += 64 * NWV)
+      prefill_block<D, HG, false, EXTRA>(k_pages, vt_pages, table, k0, kvh, n_kv, page_size, col, g, heads_here, my_pos,
+                                  my_lo, lo, hi, scale_log2, qf, acc, m, l, slope, kept, vh, n_vh);
+  }
   int kb = (lo / 64) * 64 + 64 * wave;
   for (; kb <= hi && kb < lo_all; kb += 64 * NWV)
     prefill_block<D, HG, false, EXTRA>(k_pages, vt_pages, table, kb, kvh, n_kv, page_size, col, g, heads_here, my_pos,
-                                my_lo, lo, hi, scale_log2, qf, acc, m, l, slope);
+                                my_lo, lo, hi, scale_log2, qf, acc, m, l, slope, kept, vh, n_vh);
   for (; kb + 63 <= p0; kb += 64 * NWV)
     prefill_block<D, HG, true, EXTRA>(k_pages, vt_pages, table, kb, kvh, n_kv, page_size, col, g, heads_here, my_pos,
-                               my_lo, lo, hi, scale_log2, qf, acc, m, l, slope);
+                               my_lo, lo, hi, scale_log2, qf, acc, m, l, slope, kept, vh, n_vh);
   for (; kb <= hi; kb += 64 * NWV)
     prefill_block<D, HG, false, EXTRA>(k_pages, vt_pages, table, kb, kvh, n_kv, page_size, col, g, heads_here, my_pos,
-                                my_lo, lo, hi, scale_log2, qf, acc, m, l, slope);
+                                my_lo, lo, hi, scale_log2, qf, acc, m, l, slope, kept, vh, n_vh);
   if (NWV > 1) {
     // Waves 1.. hand their state to wave 0: maximum, sum and the output accumulators of each head.
     if (wave > 0) {
@@ -327,6 +344,8 @@ struct PrefillExtras {       // what the plain form does not have: see ta_prefil
   int chunk;
   const float* slopes;
   const float* sinks;
+  int keep_first;            // with a window: keys below this stay visible behind it
+  int n_v;                   // value heads in the value pages (0 or n_kv: one a key head)
 };
 
 template <int D, int HG, int NWV>
@@ -340,8 +359,9 @@ static int launch_prefill_waves(const void* q, int q_stride, void* out, const vo
 #define GO(EE) prefill_attention_kernel<D, HG, NWV, EE><<<(unsigned)workgroups, NWV * WAVE, 0, stream>>>( \
       (const bf16_t*)q, q_stride, (bf16_t*)out, (const bf16_t*)k_pages, (const bf16_t*)vt_pages, (const int*)tiles, \
       n_tiles, (const int*)cu_q, (const int*)first_position, (const int*)block_table, table_stride, n_q, n_kv, page_size, \
-      window, scale * 1.4426950408889634f, extra.chunk, extra.slopes, extra.sinks, 1.0f / scale)
-  if (extra.chunk > 0 || extra.slopes || extra.sinks) GO(true); else GO(false);
+      window, scale * 1.4426950408889634f, extra.chunk, extra.slopes, extra.sinks, 1.0f / scale, extra.keep_first, extra.n_v)
+  if (extra.chunk > 0 || extra.slopes || extra.sinks || extra.keep_first > 0 || (extra.n_v > 0 && extra.n_v < n_kv)) GO(true);
+  else GO(false);
 #undef GO
   return LAUNCH_STATUS();
 }
@@ -425,18 +445,22 @@ extern "C" int ta_prefill_attention_key_splits(int n_tiles, int n_q, int n_kv, i
 // a tile's keys (null: the keys are not cut).
 // chunk > 0: a token sees only the keys of its own run of `chunk` positions (runs counted from position 0); slopes
 // (float [n_q] or null): head h's score loses slopes[h] per position of distance; sinks (float [n_q] or null): exp(sinks[h])
-// joins the softmax's denominator.  With any of the three the per-wave kernel runs, and the keys are not cut.
+// joins the softmax's denominator.  keep_first > 0 (with a window): keys at positions below it stay visible behind the
+// window; n_v (a divisor of n_kv): the value pages hold n_v heads, key head g reads value head g / (n_kv / n_v).
+// With any of these the per-wave kernel runs, and the keys are not cut.
 extern "C" int ta_prefill_attention_bf16(const void* q, int q_stride, void* out, const void* k_pages,
                                          const void* vt_pages, const void* tiles, int n_tiles, const void* cu_q,
                                          const void* first_position, const void* block_table, int table_stride,
                                          int n_q, int n_kv, int d, int page_size, int window, float scale,
                                          int shared_shape, int max_keys, int waves, int shared,
                                          void* part_o, void* part_ml, int chunk, const void* slopes, const void* sinks,
-                                         hipStream_t stream) {
+                                         int keep_first, int n_v, hipStream_t stream) {
   if (n_tiles <= 0) return 0;
   if (n_kv <= 0 || n_q % n_kv || page_size % 16 || scale == 0.f) return -1;
-  const PrefillExtras extra = {chunk, (const float*)slopes, (const float*)sinks};
-  const bool plain = chunk <= 0 && !slopes && !sinks;
+  if (n_v <= 0) n_v = n_kv;
+  if (n_kv % n_v || keep_first < 0 || (keep_first > 0 && (window < 0 || chunk > 0 || slopes))) return -1;
+  const PrefillExtras extra = {chunk, (const float*)slopes, (const float*)sinks, keep_first, n_v};
+  const bool plain = chunk <= 0 && !slopes && !sinks && keep_first == 0 && n_v == n_kv;
   const int shape = plain ? shared_shape_for(n_tiles, n_q, n_kv, d, window, shared_shape, max_keys, waves, shared) : 0;
   if (shape) {
     const int parts = (part_o && part_ml)

@@ -516,11 +516,14 @@ class Ops:
             _need(max_position // page_size < block_table.shape[1], "block table is too narrow for the positions")
         # The matrix-core kernels take chunks, slopes and sinks as they are; value heads of another size than the key
         # heads go to the generic kernel.
+        plain = plain and keep_first == 0 and value_heads == n_kv
         if (value_dim == head_dim and qkv.dtype == torch.bfloat16 and head_dim in self.DECODE_HEAD_DIMS and page_size % 16 == 0
-                and qkv.shape[1] % 8 == 0 and self.use_fast_attention and keep_first == 0 and value_heads == n_kv):
+                and qkv.shape[1] % 8 == 0 and self.use_fast_attention
+                and (keep_first == 0 or (chunk is None and slopes is None))):
             args = (qkv, out, k_pages, v_pages, positions, entry_of_token, block_table, n_q, n_kv, head_dim,
                     page_size, window, scale, max_position)
-            extras = {} if plain else dict(chunk=chunk, slopes=slopes, sinks=sinks)
+            extras = {} if plain else dict(chunk=chunk, slopes=slopes, sinks=sinks, keep_first=keep_first,
+                                           value_heads=value_heads)
             if batch is None:
                 return self._decode_attention(*args, **extras)
             if batch.q_tiles.numel() == 0:
@@ -544,7 +547,7 @@ class Ops:
                 n_tiles, _ptr(batch.cu_q), _ptr(batch.first_position), _ptr(block_table),
                 block_table.shape[1], n_q, n_kv, head_dim, page_size, choice[0], ctypes.c_float(scale), *choice[1:],
                 _ptr(part_o), _ptr(part_ml), 0 if chunk is None else int(chunk), _ptr(slopes), _ptr(sinks),
-                self._stream()), "prefill_attention")
+                keep_first, value_heads, self._stream()), "prefill_attention")
             if batch.decode_rows.numel():
                 self._decode_attention(*args, rows=batch.decode_rows, **extras)
             return out
@@ -571,8 +574,9 @@ class Ops:
 
     def _decode_attention(self, qkv, out, k_pages, v_pages, positions, entry_of_token, block_table,
                           n_q, n_kv, head_dim, page_size, window, scale, max_position, rows=None,
-                          identity_entries=False, chunk=None, slopes=None, sinks=None):
-        """Matrix-core attention of single tokens with the key range split over workgroups."""
+                          identity_entries=False, chunk=None, slopes=None, sinks=None, keep_first=0, value_heads=None):
+        """Matrix-core attention of single tokens with the key range split over workgroups (kept first keys behind a
+        window are further splits of their own)."""
         n_items = qkv.shape[0] if rows is None else rows.numel()
         max_keys = (block_table.shape[1] * page_size) if max_position is None else max_position + 1
         # The split is planned for the context rounded up to a multiple of 512 keys: a step that replays a
@@ -587,6 +591,8 @@ class Ops:
         split_keys = max(self.min_split_keys, -(-max_keys // per_split))
         split_keys = -(-split_keys // 32) * 32
         splits = max(1, -(-(max_keys + 31) // split_keys))
+        kept_splits = -(-int(keep_first) // split_keys) if keep_first and window is not None else 0
+        splits += kept_splits
         part_o = part_ml = None
         if splits > 1:
             part_o = torch.empty((n_items, n_q, splits, head_dim), dtype=torch.float32, device=qkv.device)
@@ -596,8 +602,9 @@ class Ops:
             _ptr(None if identity_entries and rows is None else entry_of_token), _ptr(block_table),
             block_table.shape[1], _ptr(part_o), _ptr(part_ml), n_items,
             n_q, n_kv, head_dim, page_size, -1 if window is None else int(window), ctypes.c_float(scale),
-            split_keys, splits, 0 if chunk is None else int(chunk), _ptr(slopes), _ptr(sinks), self._stream()),
-            "decode_attention")
+            split_keys, splits, 0 if chunk is None else int(chunk), _ptr(slopes), _ptr(sinks),
+            int(keep_first) if kept_splits else 0, kept_splits, n_kv if value_heads is None else int(value_heads),
+            self._stream()), "decode_attention")
         return out
 
     # --------------------------------------------------------------------- linear
