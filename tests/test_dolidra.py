@@ -548,6 +548,28 @@ def test_the_token_input_and_the_tanh_gelu_gate(backend, dim, columns):
     stream = torch.zeros((tokens, width), dtype=torch.float32, device=device)
     ops.norm_add_rmsnorm(stream, y, dev(w["norm"], torch.float32), eps, None, 0.0, torch.empty_like(y))
     assert float((stream.double().cpu() - want).abs().max()) <= tolerance(dtype, 3e-5, 5e-2) * float(want.abs().max())
+    # The same in one kernel with the norm behind the sub-layer before it and the norm of the next one behind it.
+    if hasattr(ops, "norm_side_norm"):
+        delta, behind, nxt = rounded(5 * rand(tokens, width), dtype), rand(width).float().double(), rand(width).float().double()
+        first = x + plain.weighted_norm(delta, behind, 3e-5)
+        after = first + plain.token_side_input(first, ids, table, w, layer, dim, eps)
+        stream = dev(x, torch.float32)
+        out = torch.empty((tokens, width), dtype=dtype, device=device)
+        done = ops.norm_side_norm(stream, dev(delta), dev(behind, torch.float32), 3e-5, dev(pad(w["gate"], columns, width)),
+                                  dev(pad(w["proj"], width, columns)), dev(w["norm"], torch.float32), eps, dev(table),
+                                  dev(ids, torch.int32), layer * dim, dim, dev(nxt, torch.float32), 1e-6, out)
+        assert done is out
+        assert float((stream.double().cpu() - after).abs().max()) <= tolerance(dtype, 3e-5, 5e-2) * float(after.abs().max())
+        want_rows = plain.weighted_norm(after, nxt, 1e-6)
+        assert float((out.double().cpu() - want_rows).abs().max()) <= tolerance(dtype, 3e-5, 5e-2) * float(want_rows.abs().max())
+        picked = torch.tensor([4, 1], dtype=torch.int32, device=device)            # a subset of rows stores nothing
+        stream = dev(x, torch.float32)
+        out = torch.empty((2, width), dtype=dtype, device=device)
+        ops.norm_side_norm(stream, dev(delta), dev(behind, torch.float32), 3e-5, dev(pad(w["gate"], columns, width)),
+                           dev(pad(w["proj"], width, columns)), dev(w["norm"], torch.float32), eps, dev(table),
+                           dev(ids, torch.int32), layer * dim, dim, dev(nxt, torch.float32), 1e-6, out, picked)
+        assert torch.equal(stream.cpu(), x.float())
+        assert float((out.double().cpu() - want_rows[[4, 1]]).abs().max()) <= tolerance(dtype, 3e-5, 5e-2) * float(want_rows.abs().max())
     # The dense feed-forward's activation.
     gate_up = rounded(3 * rand(tokens, 2 * 22), dtype)
     out = torch.empty((tokens, 22), dtype=dtype, device=device)

@@ -99,6 +99,132 @@ norm_add_rmsnorm_long_kernel(float* __restrict__ residual, const TD* __restrict_
   }
 }
 
+#define NA_MAX_SIDE 64     // the widest per-layer token input the fused kernel takes
+
+__device__ __forceinline__ float na_gelu_tanh(float z) {
+  return 0.5f * z * (1.0f + tanhf(0.7978845608028654f * (z + 0.044715f * z * z * z)));
+}
+
+// The same with a token input between the two norms: with x the stream after the first add,
+//   g[j] = gelu_tanh(gate[j, :] . x) * table[token, offset + j]  (j < dim),  y = proj g,
+//   x += y / sqrt(mean(y^2) + side_eps) * side_norm,
+// and then the norm before the next sub-layer.  gate [>= dim, hidden], proj [hidden, proj_stride] (its first dim
+// columns count), table [vocab, table_width] and delta have the type T; the stream, the dot products and the norms are float.
+template <typename T>
+__global__ void __launch_bounds__(NA_THREADS)
+norm_side_norm_kernel(float* __restrict__ residual, const T* __restrict__ delta, const float* __restrict__ post_weight,
+                      float post_eps, const T* __restrict__ gate, const T* __restrict__ proj, int proj_stride,
+                      const float* __restrict__ side_norm, float side_eps, const T* __restrict__ table, int table_width,
+                      const int* __restrict__ token_ids, int offset, int dim, const float* __restrict__ weight, float eps,
+                      T* __restrict__ out, const int* __restrict__ rows, int hidden, int store_residual) {
+  __shared__ float scratch[16];
+  __shared__ float part_s[NA_THREADS / WAVE][NA_MAX_SIDE];
+  __shared__ float g_s[NA_MAX_SIDE];
+  const int i = blockIdx.x;
+  const int r = rows ? rows[i] : i;
+  const int lane = threadIdx.x & (WAVE - 1), wave = threadIdx.x / WAVE;
+  float* res = residual + (size_t)r * hidden;
+  const T* del = delta ? delta + (size_t)r * hidden : nullptr;
+  float x[NA_PER], d[NA_PER];
+#pragma unroll
+  for (int c = 0; c < NA_PER; ++c) {
+    const int h = c * NA_THREADS + threadIdx.x;
+    x[c] = h < hidden ? res[h] : 0.f;
+    d[c] = (del && h < hidden) ? ld(del + h) : 0.f;
+  }
+  if (del) {
+    if (post_weight) {
+      float sq = 0.f;
+#pragma unroll
+      for (int c = 0; c < NA_PER; ++c) sq += d[c] * d[c];
+      const float inv = 1.0f / sqrtf(block_sum(sq, scratch) / (float)hidden + post_eps);
+#pragma unroll
+      for (int c = 0; c < NA_PER; ++c) {
+        const int h = c * NA_THREADS + threadIdx.x;
+        if (h < hidden) d[c] = d[c] * inv * post_weight[h];
+      }
+    }
+#pragma unroll
+    for (int c = 0; c < NA_PER; ++c) x[c] += d[c];
+  }
+  // The gate's dot products: every thread's share of each, summed over the wave, then over the waves through LDS.
+  const int chunks = (hidden + NA_THREADS - 1) / NA_THREADS;
+  for (int j = 0; j < dim; ++j) {
+    const T* row = gate + (size_t)j * hidden;
+    float part = 0.f;
+#pragma unroll
+    for (int c = 0; c < NA_PER; ++c) {
+      const int h = c * NA_THREADS + threadIdx.x;
+      if (c < chunks && h < hidden) part = fmaf(ld(row + h), x[c], part);
+    }
+    part = wave_sum(part);
+    if (lane == 0) part_s[wave][j] = part;
+  }
+  __syncthreads();
+  if (threadIdx.x < dim) {
+    float z = 0.f;
+#pragma unroll
+    for (int w = 0; w < NA_THREADS / WAVE; ++w) z += part_s[w][threadIdx.x];
+    g_s[threadIdx.x] = na_gelu_tanh(z) * ld(table + (size_t)token_ids[r] * table_width + offset + threadIdx.x);
+  }
+  __syncthreads();
+  float y[NA_PER], sq = 0.f;
+#pragma unroll
+  for (int c = 0; c < NA_PER; ++c) {
+    const int h = c * NA_THREADS + threadIdx.x;
+    y[c] = 0.f;
+    if (c < chunks && h < hidden) {
+      const T* row = proj + (size_t)h * proj_stride;
+      float sum = 0.f;
+      for (int j = 0; j < dim; ++j) sum = fmaf(ld(row + j), g_s[j], sum);
+      y[c] = sum;
+    }
+    sq += y[c] * y[c];
+  }
+  const float inv_y = 1.0f / sqrtf(block_sum(sq, scratch) / (float)hidden + side_eps);
+  sq = 0.f;
+#pragma unroll
+  for (int c = 0; c < NA_PER; ++c) {
+    const int h = c * NA_THREADS + threadIdx.x;
+    if (h < hidden) {
+      x[c] += y[c] * inv_y * side_norm[h];
+      if (store_residual) res[h] = x[c];
+    }
+    sq += x[c] * x[c];
+  }
+  float inv = 1.f;
+  if (weight) inv = 1.0f / sqrtf(block_sum(sq, scratch) / (float)hidden + eps);
+  T* dst = out + (size_t)i * hidden;
+#pragma unroll
+  for (int c = 0; c < NA_PER; ++c) {
+    const int h = c * NA_THREADS + threadIdx.x;
+    if (h < hidden) st(dst + h, weight ? x[c] * inv * weight[h] : x[c]);
+  }
+}
+
+// dtype: of delta, gate, proj, table and out.  Returns -2 for sizes the fused kernel does not take (rows longer than
+// a workgroup holds, a wider token input): the caller then runs the steps one by one.
+extern "C" int ta_norm_side_norm(void* residual, const void* delta, const void* post_weight, float post_eps, const void* gate,
+                                 const void* proj, int proj_stride, const void* side_norm, float side_eps, const void* table,
+                                 int table_width, const void* token_ids, int offset, int dim, const void* weight, float eps,
+                                 void* out, const void* rows, int n_rows, int hidden, int store_residual, int dtype,
+                                 hipStream_t stream) {
+  if (n_rows <= 0) return 0;
+  if (hidden <= 0 || hidden > NA_THREADS * NA_PER || dim <= 0 || dim > NA_MAX_SIDE) return -2;
+  if (offset < 0 || offset + dim > table_width || proj_stride < dim) return -1;
+  if (dtype == DT_F32)
+    norm_side_norm_kernel<float><<<n_rows, NA_THREADS, 0, stream>>>(
+        (float*)residual, (const float*)delta, (const float*)post_weight, post_eps, (const float*)gate, (const float*)proj,
+        proj_stride, (const float*)side_norm, side_eps, (const float*)table, table_width, (const int*)token_ids, offset, dim,
+        (const float*)weight, eps, (float*)out, (const int*)rows, hidden, store_residual);
+  else
+    norm_side_norm_kernel<bf16_t><<<n_rows, NA_THREADS, 0, stream>>>(
+        (float*)residual, (const bf16_t*)delta, (const float*)post_weight, post_eps, (const bf16_t*)gate, (const bf16_t*)proj,
+        proj_stride, (const float*)side_norm, side_eps, (const bf16_t*)table, table_width, (const int*)token_ids, offset, dim,
+        (const float*)weight, eps, (bf16_t*)out, (const int*)rows, hidden, store_residual);
+  return LAUNCH_STATUS();
+}
+
 // delta_dtype, out_dtype: DT_F32 or DT_BF16 (a bfloat16 delta with a float result serves whoever wants the
 // normalised term by itself).
 extern "C" int ta_norm_add_rmsnorm(void* residual, const void* delta, const void* post_weight, float post_eps,

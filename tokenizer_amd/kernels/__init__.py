@@ -155,7 +155,7 @@ class Ops:
                      "ta_sample_workspace_words", "ta_library_gemm_bf16", "ta_compute_units", "ta_read_stream",
                      "ta_embedding_streams", "ta_streams_step", "ta_token_shift", "ta_mlstm_scan", "ta_mlstm_chunked", "ta_head_norm_gate",
                      "ta_capped_gate", "ta_norm_add_rmsnorm", "ta_norm_rotate_store", "ta_differential_heads",
-                     "ta_sigmoid_head_gate", "ta_route_top", "ta_expert_gate", "ta_side_gate", "ta_gelu_gate"):
+                     "ta_sigmoid_head_gate", "ta_route_top", "ta_expert_gate", "ta_side_gate", "ta_gelu_gate", "ta_norm_side_norm"):
             getattr(self.lib, name).restype = ctypes.c_int
         self.lib.ta_library_gemm_bf16.argtypes = [ctypes.c_void_p] * 4 + [ctypes.c_int] * 5 + [
             ctypes.c_void_p, ctypes.c_size_t, ctypes.c_int, ctypes.c_void_p]
@@ -295,6 +295,38 @@ class Ops:
                                                  _ptr(weight), ctypes.c_float(eps), _ptr(out), _ptr(rows), n_rows, hidden,
                                                  int(store_residual and delta is not None), delta_code, _code(out.dtype),
                                                  self._stream()), "norm_add_rmsnorm")
+        return out
+
+    def norm_side_norm(self, residual: torch.Tensor, delta: torch.Tensor, post_weight: torch.Tensor, post_eps: float,
+                       gate: torch.Tensor, proj: torch.Tensor, side_norm: torch.Tensor, side_eps: float, table: torch.Tensor,
+                       token_ids: torch.Tensor, offset: int, dim: int, weight: torch.Tensor | None, eps: float,
+                       out: torch.Tensor, rows: torch.Tensor | None = None):
+        """`norm_add_rmsnorm` with a token input between the add and the last norm, in one kernel: with x the stream
+        after the add, g = gelu_tanh(gate[:dim] x) * table[token, offset : offset + dim], y = proj[:, :dim] g,
+        x += y / sqrt(mean(y^2) + side_eps) * side_norm (stored back unless `rows` selects a subset), out = x /
+        sqrt(mean(x^2) + eps) * weight.  gate [>= dim, H], proj [H, >= dim], table [V, W] and delta share out's dtype.
+        Returns None for sizes the kernel does not take (rows of more than 4,096 elements, dim above 64)."""
+        _dev(residual, delta, post_weight, gate, proj, side_norm, table, token_ids, weight, out, rows)
+        hidden = residual.shape[1]
+        if hidden > 4096 or dim > 64:
+            return None
+        n_rows = residual.shape[0] if rows is None else rows.numel()
+        _need(residual.dtype == torch.float32 and residual.is_contiguous(), "the residual stream is float32")
+        _need(delta.shape == residual.shape and delta.is_contiguous() and delta.dtype == out.dtype, "delta [T, H] of out's dtype")
+        _need(tuple(out.shape) == (n_rows, hidden) and out.is_contiguous(), "norm output shape")
+        for vector in (post_weight, side_norm, weight):
+            _need(vector is None or (vector.dtype == torch.float32 and vector.numel() == hidden), "norm weights are float32 [H]")
+        _need(gate.dtype == proj.dtype == table.dtype == out.dtype and gate.is_contiguous() and proj.is_contiguous()
+              and table.is_contiguous(), "gate, proj and table are contiguous, of out's dtype")
+        _need(gate.shape[0] >= dim and gate.shape[1] == hidden and proj.shape[0] == hidden and proj.shape[1] >= dim, "gate [dim, H], proj [H, dim]")
+        _need(table.dim() == 2 and 0 <= offset and offset + dim <= table.shape[1], "the table's slice")
+        _need(token_ids.dtype == torch.int32 and token_ids.numel() == residual.shape[0], "token ids are int32 [T]")
+        _need(rows is None or rows.dtype == torch.int32, "rows are int32")
+        self._check(self.lib.ta_norm_side_norm(
+            _ptr(residual), _ptr(delta), _ptr(post_weight), ctypes.c_float(post_eps), _ptr(gate), _ptr(proj), proj.shape[1],
+            _ptr(side_norm), ctypes.c_float(side_eps), _ptr(table), table.shape[1], _ptr(token_ids), offset, dim, _ptr(weight),
+            ctypes.c_float(eps), _ptr(out), _ptr(rows), n_rows, hidden, int(rows is None), _code(out.dtype), self._stream()),
+            "norm_side_norm")
         return out
 
     def norm_rotate_store(self, qkv: torch.Tensor, bias: torch.Tensor | None, positions: torch.Tensor,

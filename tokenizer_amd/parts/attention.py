@@ -102,20 +102,23 @@ class GQAttention(Mixer):
         self.gate_offset = sum(part.shape[0] for part in joined)
         if spec.head_gate:
             joined.append(tensors["gate_proj.weight"])
+        # (Rows of the joined product in eights: the matrix-core attention kernels read a row sixteen bytes at a time.)
+        fill = (-sum(part.shape[0] for part in joined)) % 8 if runtime.dtype == torch.bfloat16 else 0
+        if fill:
+            joined.append(q.new_zeros((fill, hidden)))
         self.w_qkv = torch.cat(joined, dim=0).contiguous()
         self.b_qkv = None
         if spec.qkv_bias:
             bias = [by_kv_head(tensors["q_proj.bias"]) if self.maps > 1 else tensors["q_proj.bias"],
                     tensors["k_proj.bias"], tensors["v_proj.bias"]]
-            if spec.head_gate:
-                bias.append(bias[0].new_zeros(H))
+            bias.append(bias[0].new_zeros((H if spec.head_gate else 0) + fill))
             self.b_qkv = torch.cat(bias, dim=0).contiguous()
         self.lam = None
         if spec.differential is not None:
             pair = lambda a, b: torch.exp((tensors[a].to(torch.float32) * tensors[b].to(torch.float32)).sum())
             self.lam = (pair("lq1", "lk1") - pair("lq2", "lk2") + float(spec.differential)).reshape(1).contiguous()
             self.out_scale = 1.0 - float(spec.differential)
-        self.q_norm = tensors["q_norm"].to(torch.float32).contiguous() if spec.qk_norm else None
+        self.q_norm = by_kv_head(tensors["q_norm"]).to(torch.float32).contiguous() if spec.qk_norm else None
         self.k_norm = tensors["k_norm"].to(torch.float32).contiguous() if spec.qk_norm else None
         self.head_gate, self.eps = spec.head_gate, float(spec.eps)
         self.w_o, self.b_o = tensors["o_proj.weight"], None
@@ -153,8 +156,8 @@ class GQAttention(Mixer):
             for name in ("lq1", "lk1", "lq2", "lk2"):
                 out[name] = TensorSpec((spec.head_dim,), role="vector", std=0.1)
         if spec.qk_norm is not None:
-            out["q_norm"] = TensorSpec((spec.n_heads * spec.head_dim,), init="ones", role="vector")
-            out["k_norm"] = TensorSpec((spec.n_kv_heads * spec.head_dim,), init="ones", role="vector")
+            out["q_norm"] = TensorSpec((q_out,), init="ones", role="vector")
+            out["k_norm"] = TensorSpec((kv_out,), init="ones", role="vector")
         if spec.head_gate:
             out["gate_proj.weight"] = TensorSpec((spec.n_heads, hidden))
         return out

@@ -194,12 +194,20 @@ class NormedDelta:
     """What a sub-layer that is normalised behind itself hands on: its output `rows` [T, H] (compute dtype) still to
     be brought to unit RMS, scaled by `weight` (float32 [H]) and added to the stream.  A norm of the form
     x / sqrt(mean(x^2) + eps) * w takes it as its delta and does all of that in its own kernel
-    (`ops.norm_add_rmsnorm`); for anyone else `resolve()` gives the sum's term as a float32 tensor."""
+    (`ops.norm_add_rmsnorm`); for anyone else `resolve()` gives the sum's term as a float32 tensor.
 
-    def __init__(self, ops, rows: torch.Tensor, weight: torch.Tensor, eps: float):
-        self.ops, self.rows, self.weight, self.eps = ops, rows, weight, float(eps)
+    `side` (or None): something that is still to be added behind this term and depends on the stream as it then
+    stands (a block's per-layer token input): an object with `fused(residual, delta, weight, eps, out, rows)`, which
+    does the add, its own addition and the next norm in one kernel or returns None, and `settle(residual, delta)`,
+    which adds this term to the stream, works its own addition out step by step and returns it as a `NormedDelta`
+    without a `side`."""
+
+    def __init__(self, ops, rows: torch.Tensor, weight: torch.Tensor, eps: float, side=None):
+        self.ops, self.rows, self.weight, self.eps, self.side = ops, rows, weight, float(eps), side
 
     def resolve(self) -> torch.Tensor:
+        if self.side is not None:
+            raise ValueError("a term with an addition behind it that reads the stream cannot stand alone: hand it to a norm")
         zero = torch.zeros((self.rows.shape[0], self.rows.shape[1]), dtype=torch.float32, device=self.rows.device)
         out = torch.empty_like(zero)
         return self.ops.norm_add_rmsnorm(zero, self.rows, self.weight, self.eps, None, 0.0, out, store_residual=False)

@@ -95,14 +95,40 @@ class SandwichNormBlock(Block):
             out = self.feed_forward.forward(self.feed_forward_norm.apply(residual, delta), ctx)
             delta = NormedDelta(ops, out, self.after_feed_forward, self.eps)
         if self.side_dim:
-            # The stream as it stands behind the feed-forward, in the compute dtype, for the gate's product.
-            rows = torch.empty((residual.shape[0], self.width), dtype=self.runtime.dtype, device=residual.device)
-            if isinstance(delta, NormedDelta):
-                ops.norm_add_rmsnorm(residual, delta.rows, delta.weight, delta.eps, None, 0.0, rows)
+            if isinstance(delta, NormedDelta) and delta.side is None:
+                delta.side = _TokenInput(self, ctx.token_ids)     # whoever takes the term next adds the token input behind it
             else:                                   # what a block of another kind handed on: a plain sum, or nothing
-                ops.norm_add_rmsnorm(residual, None if delta is None else as_tensor(delta), None, 0.0, None, 0.0, rows)
-            gate = ops.linear(rows, self.side_gate)
-            gated = torch.empty_like(gate)
-            ops.side_gate(gate, self.side_table, ctx.token_ids, self.side_offset, self.side_dim, gated)
-            delta = NormedDelta(ops, ops.linear(gated, self.side_proj), self.side_norm, self.eps)
+                delta = _TokenInput(self, ctx.token_ids).settle(residual, delta)
         return delta
+
+
+class _TokenInput:
+    """A sandwich block's token input of one step, still to be added behind the block's last term."""
+
+    def __init__(self, block: SandwichNormBlock, token_ids):
+        self.block, self.token_ids = block, token_ids
+
+    def fused(self, residual, delta, weight, eps, out, rows):
+        """The term's norm and add, the token input and the norm `weight` in one kernel; None if the kernel library
+        has none for these sizes."""
+        block = self.block
+        run = getattr(block.runtime.ops, "norm_side_norm", None)
+        if run is None or out.dtype != delta.rows.dtype:
+            return None
+        return run(residual, delta.rows, delta.weight, delta.eps, block.side_gate, block.side_proj, block.side_norm,
+                   block.eps, block.side_table, self.token_ids, block.side_offset, block.side_dim, weight, eps, out, rows)
+
+    def settle(self, residual, delta) -> NormedDelta:
+        """Step by step: the stream as it stands behind the term (stored back), the gate's product, the gate, the
+        projection; returns the token input as a term of its own."""
+        block = self.block
+        ops = block.runtime.ops
+        rows = torch.empty((residual.shape[0], block.width), dtype=block.runtime.dtype, device=residual.device)
+        if isinstance(delta, NormedDelta):
+            ops.norm_add_rmsnorm(residual, delta.rows, delta.weight, delta.eps, None, 0.0, rows)
+        else:
+            ops.norm_add_rmsnorm(residual, None if delta is None else as_tensor(delta), None, 0.0, None, 0.0, rows)
+        gate = ops.linear(rows, block.side_gate)
+        gated = torch.empty_like(gate)
+        ops.side_gate(gate, block.side_table, self.token_ids, block.side_offset, block.side_dim, gated)
+        return NormedDelta(ops, ops.linear(gated, block.side_proj), block.side_norm, block.eps)

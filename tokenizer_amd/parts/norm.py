@@ -35,6 +35,11 @@ class RMSNorm(Norm):
         n_rows = residual.shape[0] if rows is None else rows.numel()
         out = torch.empty((n_rows, self.size), dtype=self.runtime.dtype, device=residual.device)
         if isinstance(delta, NormedDelta):
+            if delta.side is not None:
+                done = delta.side.fused(residual, delta, self.weight, self.eps, out, rows)
+                if done is not None:
+                    return done
+                delta = delta.side.settle(residual, delta)
             return self.runtime.ops.norm_add_rmsnorm(residual, delta.rows, delta.weight, delta.eps, self.weight, self.eps,
                                                      out, rows, store_residual=rows is None)
         return self.runtime.ops.add_rmsnorm(residual, delta, self.weight, self.eps, out, rows,
