@@ -53,7 +53,7 @@ template <int MB, int NW, bool GATED, typename OutT, bool ROPE = false, int NB =
 __global__ void __launch_bounds__(NW * WAVE)
 skinny_gemm_kernel(const bf16_t* __restrict__ A, int lda, int k_chunk, const bf16_t* __restrict__ W,
                    OutT* __restrict__ C, int ldc, int M, int N, int K_all, float* __restrict__ partial,
-                   const float* __restrict__ bias, const RopeStore rope = RopeStore()) {
+                   const float* __restrict__ bias, const RopeStore rope = RopeStore(), int gate_act = 0) {
   // (What the walk over K needs stands in the first fourteen words of the arguments, which are in scalar registers
   // when a wave starts; the bias and the rotation's arguments, which the epilogue needs, lie behind.)
   HELD(A, lda, k_chunk, W, C, ldc, M, N, K_all, partial);
@@ -227,7 +227,10 @@ skinny_gemm_kernel(const bf16_t* __restrict__ A, int lda, int k_chunk, const bf1
         continue;
       }
       if (bias && !partial && n + r < n_out) sum0 += bias[n + r];
-      v[r] = GATED ? sum0 / (1.0f + __expf(-sum0)) * sum1 : sum0;
+      // gate_act 1: the tanh form of GELU in place of silu.
+      v[r] = !GATED ? sum0
+             : gate_act == 1 ? 0.5f * sum0 * (1.0f + tanhf(0.7978845608028654f * (sum0 + 0.044715f * sum0 * sum0 * sum0))) * sum1
+                             : sum0 / (1.0f + __expf(-sum0)) * sum1;
     }
     if constexpr (ROPE) {
       const int d = rope.d, i = rope_first + 4 * (ln >> 4);          // elements i..i+3 of the head, and i + half
@@ -291,7 +294,7 @@ extern "C" void ta_skinny_lines(int on) { g_lines = on; }
 
 template <int MB, int NW, bool GATED, int NB = 1, bool LINES = false>
 static int launch_skinny(const void* A, int lda, const void* W, const void* bias, void* C, int ldc, int M, int N,
-                         int K, int out_dtype, hipStream_t stream, int splits = 1, void* partial = nullptr) {
+                         int K, int out_dtype, hipStream_t stream, int splits = 1, void* partial = nullptr, int gate_act = 0) {
   const int n_out = GATED ? N / 2 : N;
   const int k_chunk = splits > 1 ? ((K + splits - 1) / splits + 31) / 32 * 32 : K;
   if (splits > 1) splits = (K + k_chunk - 1) / k_chunk;          // no part without a step of its own
@@ -299,10 +302,10 @@ static int launch_skinny(const void* A, int lda, const void* W, const void* bias
   float* slabs = splits > 1 ? (float*)partial : nullptr;
   if (out_dtype == DT_F32)
     skinny_gemm_kernel<MB, NW, GATED, float, false, NB, LINES><<<grid, NW * WAVE, 0, stream>>>(
-        (const bf16_t*)A, lda, k_chunk, (const bf16_t*)W, (float*)C, ldc, M, N, K, slabs, (const float*)bias);
+        (const bf16_t*)A, lda, k_chunk, (const bf16_t*)W, (float*)C, ldc, M, N, K, slabs, (const float*)bias, RopeStore(), gate_act);
   else
     skinny_gemm_kernel<MB, NW, GATED, bf16_t, false, NB, LINES><<<grid, NW * WAVE, 0, stream>>>(
-        (const bf16_t*)A, lda, k_chunk, (const bf16_t*)W, (bf16_t*)C, ldc, M, N, K, slabs, (const float*)bias);
+        (const bf16_t*)A, lda, k_chunk, (const bf16_t*)W, (bf16_t*)C, ldc, M, N, K, slabs, (const float*)bias, RopeStore(), gate_act);
   int status = LAUNCH_STATUS();
   if (status == 0 && splits > 1 && C) status = launch_splitk_reduce(slabs, bias, C, M, N, ldc, splits, out_dtype, stream);
   return status;
@@ -310,10 +313,10 @@ static int launch_skinny(const void* A, int lda, const void* W, const void* bias
 
 template <int MB, bool GATED>
 static int pick_waves(const void* A, int lda, const void* W, const void* bias, void* C, int ldc, int M, int N,
-                      int K, int out_dtype, hipStream_t stream, int col_blocks = 0) {
+                      int K, int out_dtype, hipStream_t stream, int col_blocks = 0, int gate_act = 0) {
   if constexpr (MB >= 3) {
     if (column_blocks(col_blocks, M, GATED ? N / 2 : N, 1) == 2)
-      return launch_skinny<MB, 8, GATED, 2>(A, lda, W, bias, C, ldc, M, N, K, out_dtype, stream);
+      return launch_skinny<MB, 8, GATED, 2>(A, lda, W, bias, C, ldc, M, N, K, out_dtype, stream, 1, nullptr, gate_act);
   }
   if constexpr (MB == 1 && !GATED) {
     // Up to sixteen rows against tens of thousands of output columns (the vocabulary projection of a decode
@@ -329,20 +332,21 @@ static int pick_waves(const void* A, int lda, const void* W, const void* bias, v
   const int tiles = ((GATED ? N / 2 : N) + 15) / 16;
   const int k_steps = (K + 31) / 32;
   if (tiles >= 1024 || k_steps <= 8)
-    return launch_skinny<MB, 4, GATED>(A, lda, W, bias, C, ldc, M, N, K, out_dtype, stream);
+    return launch_skinny<MB, 4, GATED>(A, lda, W, bias, C, ldc, M, N, K, out_dtype, stream, 1, nullptr, gate_act);
   if (tiles >= 256 || k_steps <= 32 || MB * (GATED ? 2 : 1) > 2)
-    return launch_skinny<MB, 8, GATED>(A, lda, W, bias, C, ldc, M, N, K, out_dtype, stream);
-  return launch_skinny<MB, 16, GATED>(A, lda, W, bias, C, ldc, M, N, K, out_dtype, stream);
+    return launch_skinny<MB, 8, GATED>(A, lda, W, bias, C, ldc, M, N, K, out_dtype, stream, 1, nullptr, gate_act);
+  return launch_skinny<MB, 16, GATED>(A, lda, W, bias, C, ldc, M, N, K, out_dtype, stream, 1, nullptr, gate_act);
 }
 
-// M <= 64; K, lda multiples of 8; pointers 16-byte aligned; with `gated` N is even and C is [M, N/2].
+// M <= 64; K, lda multiples of 8; pointers 16-byte aligned; with `gated` N is even and C is [M, N/2]
+// (gated 1: silu(gate) * up; 2: the tanh form of GELU in place of silu).
 // col_blocks: blocks of sixteen output columns per workgroup, 0 = the launcher's choice (see column_blocks).
 extern "C" int ta_gemm_skinny_bf16(const void* A, int lda, const void* W, const void* bias, void* C, int ldc,
                                    int M, int N, int K, int out_dtype, int gated, int col_blocks, hipStream_t stream) {
   if (M <= 0 || N <= 0) return 0;
   if (M > 64 || (K & 7) || (lda & 7) || (gated && (N & 1))) return -1;
   const int mb = (M + 15) / 16;
-#define GO(MBV) (gated ? pick_waves<MBV, true>(A, lda, W, bias, C, ldc, M, N, K, out_dtype, stream, col_blocks) \
+#define GO(MBV) (gated ? pick_waves<MBV, true>(A, lda, W, bias, C, ldc, M, N, K, out_dtype, stream, col_blocks, gated == 2) \
                        : pick_waves<MBV, false>(A, lda, W, bias, C, ldc, M, N, K, out_dtype, stream, col_blocks))
   switch (mb) {
     case 1: return GO(1);

@@ -23,12 +23,16 @@ norm_add_rmsnorm_kernel(float* __restrict__ residual, const TD* __restrict__ del
   const int r = rows ? rows[i] : i;
   float* res = residual + (size_t)r * hidden;
   const TD* del = delta ? delta + (size_t)r * hidden : nullptr;
-  float x[NA_PER], d[NA_PER];
+  // Everything a thread needs of the rows and the two weights is asked for at the start: one trip to memory.
+  float x[NA_PER], d[NA_PER], behind_w[NA_PER], next_w[NA_PER];
 #pragma unroll
   for (int c = 0; c < NA_PER; ++c) {
     const int h = c * NA_THREADS + threadIdx.x;
-    x[c] = h < hidden ? res[h] : 0.f;
-    d[c] = (del && h < hidden) ? ld(del + h) : 0.f;
+    const bool in = h < hidden;
+    x[c] = in ? res[h] : 0.f;
+    d[c] = (del && in) ? ld(del + h) : 0.f;
+    behind_w[c] = (del && post_weight && in) ? post_weight[h] : 1.f;
+    next_w[c] = (weight && in) ? weight[h] : 1.f;
   }
   if (del) {
     if (post_weight) {
@@ -37,10 +41,7 @@ norm_add_rmsnorm_kernel(float* __restrict__ residual, const TD* __restrict__ del
       for (int c = 0; c < NA_PER; ++c) sq += d[c] * d[c];
       const float inv = 1.0f / sqrtf(block_sum(sq, scratch) / (float)hidden + post_eps);
 #pragma unroll
-      for (int c = 0; c < NA_PER; ++c) {
-        const int h = c * NA_THREADS + threadIdx.x;
-        if (h < hidden) d[c] = d[c] * inv * post_weight[h];
-      }
+      for (int c = 0; c < NA_PER; ++c) d[c] *= inv * behind_w[c];
     }
 #pragma unroll
     for (int c = 0; c < NA_PER; ++c) {
@@ -60,7 +61,7 @@ norm_add_rmsnorm_kernel(float* __restrict__ residual, const TD* __restrict__ del
 #pragma unroll
   for (int c = 0; c < NA_PER; ++c) {
     const int h = c * NA_THREADS + threadIdx.x;
-    if (h < hidden) na_store(dst + h, weight ? x[c] * inv * weight[h] : x[c]);
+    if (h < hidden) na_store(dst + h, x[c] * inv * next_w[c]);
   }
 }
 
@@ -202,6 +203,149 @@ norm_side_norm_kernel(float* __restrict__ residual, const T* __restrict__ delta,
   }
 }
 
+// Sixteen bytes of a row as floats: eight bfloat16 or four float elements.
+template <typename T> struct NaVec;
+template <> struct NaVec<bf16_t> {
+  static constexpr int N = 8;
+  __device__ static __forceinline__ void load(const bf16_t* p, float (&v)[8]) {
+    const uint4 raw = *reinterpret_cast<const uint4*>(p);
+    const uint32_t w[4] = {raw.x, raw.y, raw.z, raw.w};
+#pragma unroll
+    for (int i = 0; i < 4; ++i) { v[2 * i] = __uint_as_float(w[i] << 16); v[2 * i + 1] = __uint_as_float(w[i] & 0xffff0000u); }
+  }
+};
+template <> struct NaVec<float> {
+  static constexpr int N = 4;
+  __device__ static __forceinline__ void load(const float* p, float (&v)[4]) {
+    const float4 raw = *reinterpret_cast<const float4*>(p);
+    v[0] = raw.x; v[1] = raw.y; v[2] = raw.z; v[3] = raw.w;
+  }
+};
+
+#define NA_SIDE_PER_WAVE (NA_MAX_SIDE / (NA_THREADS / WAVE))
+
+// The same for rows, token inputs and projections in whole pieces of sixteen bytes (hidden, dim and proj_stride
+// multiples of 8 for bfloat16, of 4 for float).  The stream after the first add goes through LDS; wave w forms the
+// gate's dot products j = w, w + 4, ..., sixteen bytes of each row a lane and step, all rows of a step asked for at
+// once; the projection's rows are read the same way, all of a thread's rows a step.
+template <typename T>
+__global__ void __launch_bounds__(NA_THREADS)
+norm_side_norm_vec_kernel(float* __restrict__ residual, const T* __restrict__ delta, const float* __restrict__ post_weight,
+                          float post_eps, const T* __restrict__ gate, const T* __restrict__ proj, int proj_stride,
+                          const float* __restrict__ side_norm, float side_eps, const T* __restrict__ table, int table_width,
+                          const int* __restrict__ token_ids, int offset, int dim, const float* __restrict__ weight, float eps,
+                          T* __restrict__ out, const int* __restrict__ rows, int hidden, int store_residual) {
+  constexpr int N = NaVec<T>::N;
+  __shared__ float scratch[16];
+  __shared__ float x_s[NA_THREADS * NA_PER];
+  __shared__ float g_s[NA_MAX_SIDE];
+  const int i = blockIdx.x;
+  const int r = rows ? rows[i] : i;
+  const int lane = threadIdx.x & (WAVE - 1), wave = threadIdx.x / WAVE;
+  float* res = residual + (size_t)r * hidden;
+  const T* del = delta ? delta + (size_t)r * hidden : nullptr;
+  // The token's slice of the table is asked for now; it is used behind the dot products.
+  float e = 0.f;
+  if (threadIdx.x < dim) e = ld(table + (size_t)token_ids[r] * table_width + offset + threadIdx.x);
+  // Everything a thread needs of the rows and the three weights is asked for at the start.
+  float x[NA_PER], d[NA_PER], behind_w[NA_PER], tail_w[NA_PER], next_w[NA_PER];
+#pragma unroll
+  for (int c = 0; c < NA_PER; ++c) {
+    const int h = c * NA_THREADS + threadIdx.x;
+    const bool in = h < hidden;
+    x[c] = in ? res[h] : 0.f;
+    d[c] = (del && in) ? ld(del + h) : 0.f;
+    behind_w[c] = (del && post_weight && in) ? post_weight[h] : 1.f;
+    tail_w[c] = in ? side_norm[h] : 0.f;
+    next_w[c] = (weight && in) ? weight[h] : 0.f;
+  }
+  if (del) {
+    if (post_weight) {
+      float sq = 0.f;
+#pragma unroll
+      for (int c = 0; c < NA_PER; ++c) sq += d[c] * d[c];
+      const float inv = 1.0f / sqrtf(block_sum(sq, scratch) / (float)hidden + post_eps);
+#pragma unroll
+      for (int c = 0; c < NA_PER; ++c) d[c] *= inv * behind_w[c];
+    }
+#pragma unroll
+    for (int c = 0; c < NA_PER; ++c) x[c] += d[c];
+  }
+#pragma unroll
+  for (int c = 0; c < NA_PER; ++c) {
+    const int h = c * NA_THREADS + threadIdx.x;
+    if (h < hidden) x_s[h] = x[c];
+  }
+  __syncthreads();
+  float acc[NA_SIDE_PER_WAVE];
+#pragma unroll
+  for (int jj = 0; jj < NA_SIDE_PER_WAVE; ++jj) acc[jj] = 0.f;
+  for (int at = lane * N; at < hidden; at += WAVE * N) {
+    float xv[N];
+#pragma unroll
+    for (int k = 0; k < N; ++k) xv[k] = x_s[at + k];
+#pragma unroll
+    for (int jj = 0; jj < NA_SIDE_PER_WAVE; ++jj) {
+      const int j = wave + (NA_THREADS / WAVE) * jj;
+      if (j < dim) {
+        float gv[N];
+        NaVec<T>::load(gate + (size_t)j * hidden + at, gv);
+#pragma unroll
+        for (int k = 0; k < N; ++k) acc[jj] = fmaf(gv[k], xv[k], acc[jj]);
+      }
+    }
+  }
+#pragma unroll
+  for (int jj = 0; jj < NA_SIDE_PER_WAVE; ++jj) {
+    const int j = wave + (NA_THREADS / WAVE) * jj;
+    const float z = wave_sum(acc[jj]);
+    if (lane == 0 && j < dim) g_s[j] = z;
+  }
+  __syncthreads();
+  if (threadIdx.x < dim) g_s[threadIdx.x] = na_gelu_tanh(g_s[threadIdx.x]) * e;
+  __syncthreads();
+  float y[NA_PER];
+#pragma unroll
+  for (int c = 0; c < NA_PER; ++c) y[c] = 0.f;
+  for (int at = 0; at < dim; at += N) {
+    float gv[N];
+#pragma unroll
+    for (int k = 0; k < N; ++k) gv[k] = g_s[at + k];
+#pragma unroll
+    for (int c = 0; c < NA_PER; ++c) {
+      const int h = c * NA_THREADS + threadIdx.x;
+      if (h < hidden) {
+        float pv[N];
+        NaVec<T>::load(proj + (size_t)h * proj_stride + at, pv);
+#pragma unroll
+        for (int k = 0; k < N; ++k) y[c] = fmaf(pv[k], gv[k], y[c]);
+      }
+    }
+  }
+  float sq = 0.f;
+#pragma unroll
+  for (int c = 0; c < NA_PER; ++c) sq += y[c] * y[c];
+  const float inv_y = 1.0f / sqrtf(block_sum(sq, scratch) / (float)hidden + side_eps);
+  sq = 0.f;
+#pragma unroll
+  for (int c = 0; c < NA_PER; ++c) {
+    const int h = c * NA_THREADS + threadIdx.x;
+    if (h < hidden) {
+      x[c] += y[c] * inv_y * tail_w[c];
+      if (store_residual) res[h] = x[c];
+    }
+    sq += x[c] * x[c];
+  }
+  float inv = 1.f;
+  if (weight) inv = 1.0f / sqrtf(block_sum(sq, scratch) / (float)hidden + eps);
+  T* dst = out + (size_t)i * hidden;
+#pragma unroll
+  for (int c = 0; c < NA_PER; ++c) {
+    const int h = c * NA_THREADS + threadIdx.x;
+    if (h < hidden) st(dst + h, weight ? x[c] * inv * next_w[c] : x[c]);
+  }
+}
+
 // dtype: of delta, gate, proj, table and out.  Returns -2 for sizes the fused kernel does not take (rows longer than
 // a workgroup holds, a wider token input): the caller then runs the steps one by one.
 extern "C" int ta_norm_side_norm(void* residual, const void* delta, const void* post_weight, float post_eps, const void* gate,
@@ -212,6 +356,21 @@ extern "C" int ta_norm_side_norm(void* residual, const void* delta, const void* 
   if (n_rows <= 0) return 0;
   if (hidden <= 0 || hidden > NA_THREADS * NA_PER || dim <= 0 || dim > NA_MAX_SIDE) return -2;
   if (offset < 0 || offset + dim > table_width || proj_stride < dim) return -1;
+  const int piece = dtype == DT_F32 ? 4 : 8;
+  if (hidden % piece == 0 && dim % piece == 0 && proj_stride % piece == 0 &&
+      (((uintptr_t)gate | (uintptr_t)proj) & 15) == 0) {
+    if (dtype == DT_F32)
+      norm_side_norm_vec_kernel<float><<<n_rows, NA_THREADS, 0, stream>>>(
+          (float*)residual, (const float*)delta, (const float*)post_weight, post_eps, (const float*)gate, (const float*)proj,
+          proj_stride, (const float*)side_norm, side_eps, (const float*)table, table_width, (const int*)token_ids, offset, dim,
+          (const float*)weight, eps, (float*)out, (const int*)rows, hidden, store_residual);
+    else
+      norm_side_norm_vec_kernel<bf16_t><<<n_rows, NA_THREADS, 0, stream>>>(
+          (float*)residual, (const bf16_t*)delta, (const float*)post_weight, post_eps, (const bf16_t*)gate, (const bf16_t*)proj,
+          proj_stride, (const float*)side_norm, side_eps, (const bf16_t*)table, table_width, (const int*)token_ids, offset, dim,
+          (const float*)weight, eps, (bf16_t*)out, (const int*)rows, hidden, store_residual);
+    return LAUNCH_STATUS();
+  }
   if (dtype == DT_F32)
     norm_side_norm_kernel<float><<<n_rows, NA_THREADS, 0, stream>>>(
         (float*)residual, (const float*)delta, (const float*)post_weight, post_eps, (const float*)gate, (const float*)proj,

@@ -831,9 +831,9 @@ class Ops:
         if out is None:
             out = torch.empty((m, inner), dtype=x.dtype, device=x.device)
         _need(tuple(out.shape) == (m, inner) and out.dtype == x.dtype and out.is_contiguous(), "gated output shape")
-        if act is not None:
+        if act is not None and act != "gelu_tanh":
             return self.silu_gate(self.linear(x, weight), out, act=act)
-        if (x.dtype == torch.bfloat16 and m <= self.SKINNY_ROWS
+        if (x.dtype == torch.bfloat16 and m <= self.SKINNY_ROWS and x.shape[1] % 8 == 0 and (m == 1 or x.stride(0) % 8 == 0)
                 and not (self.use_library_gemm and m > self.FUSED_ROWS
                          and weight.shape[0] * weight.shape[1] >= self.GATED_LIBRARY_WEIGHT)):
             _need(x.is_cuda and weight.is_cuda and x.dim() == 2 and x.shape[1] == weight.shape[1], "linear shapes do not fit")
@@ -843,10 +843,10 @@ class Ops:
             _need(k % 8 == 0 and lda % 8 == 0, "bfloat16 products need K and the row stride to be multiples of 8")
             _need(x.data_ptr() % 16 == 0 and weight.data_ptr() % 16 == 0, "operands must be 16-byte aligned")
             self._check(self.lib.ta_gemm_skinny_bf16(_ptr(x), lda, _ptr(weight), None, _ptr(out), inner, m, 2 * inner,
-                                                     k, _BF16, 1, self.skinny_column_blocks, self._stream()),
-                        "linear_silu_gate")
+                                                     k, _BF16, 2 if act == "gelu_tanh" else 1, self.skinny_column_blocks,
+                                                     self._stream()), "linear_silu_gate")
             return out
-        return self.silu_gate(self.linear(x, weight), out)
+        return self.silu_gate(self.linear(x, weight), out, act=act)
 
     # ------------------------------------------------------- fused decode products
     FUSED_ROWS = 16
