@@ -102,6 +102,69 @@ __global__ void gelu_gate_kernel(const T* __restrict__ in, T* __restrict__ out, 
   }
 }
 
+// Eight bfloat16 elements (sixteen bytes) as floats, and back.
+__device__ __forceinline__ void rt_unpack8(const uint4 raw, float (&v)[8]) {
+  const uint32_t w[4] = {raw.x, raw.y, raw.z, raw.w};
+#pragma unroll
+  for (int i = 0; i < 4; ++i) { v[2 * i] = __uint_as_float(w[i] << 16); v[2 * i + 1] = __uint_as_float(w[i] & 0xffff0000u); }
+}
+__device__ __forceinline__ uint4 rt_pack8(const float (&v)[8]) {
+  uint32_t w[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) w[i] = (uint32_t)float_to_bf16_bits(v[2 * i]) | ((uint32_t)float_to_bf16_bits(v[2 * i + 1]) << 16);
+  return make_uint4(w[0], w[1], w[2], w[3]);
+}
+
+// expert_gate for bfloat16 with inner, shared and columns multiples of 8: a thread makes eight columns, which lie in
+// one expert; the rows of experts a token did not choose are not read.
+__global__ void expert_gate_vec_kernel(const bf16_t* __restrict__ gate_up, const int* __restrict__ chosen,
+                                       const float* __restrict__ weights, int top, int n_experts, int inner, int shared,
+                                       int columns, bf16_t* __restrict__ out, size_t total8) {
+  const int in_stride = n_experts * 2 * inner + 2 * shared, columns8 = columns / 8;
+  for (size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x; idx < total8; idx += (size_t)gridDim.x * blockDim.x) {
+    const size_t t = idx / columns8;
+    const int c = (int)(idx - t * columns8) * 8;
+    const bf16_t* row = gate_up + t * in_stride;
+    const bf16_t* g_at = nullptr;
+    int up_off = 0;
+    float w = 0.f;
+    if (c < n_experts * inner) {
+      const int e = c / inner, i = c - e * inner;
+      for (int k = 0; k < top; ++k)
+        if (chosen[t * top + k] == e) w += weights[t * top + k];
+      if (w != 0.f) { g_at = row + (size_t)e * 2 * inner + i; up_off = inner; }
+    } else if (c < n_experts * inner + shared) {
+      g_at = row + (size_t)n_experts * 2 * inner + (c - n_experts * inner);
+      up_off = shared;
+      w = 1.f;
+    }
+    uint4 packed = make_uint4(0, 0, 0, 0);
+    if (g_at) {
+      float g[8], u[8], v[8];
+      rt_unpack8(*reinterpret_cast<const uint4*>(g_at), g);
+      rt_unpack8(*reinterpret_cast<const uint4*>(g_at + up_off), u);
+#pragma unroll
+      for (int k = 0; k < 8; ++k) v[k] = w * (g[k] / (1.0f + expf(-g[k])) * u[k]);
+      packed = rt_pack8(v);
+    }
+    *reinterpret_cast<uint4*>(out + t * columns + c) = packed;
+  }
+}
+
+// gelu_gate for bfloat16 rows whose length is a multiple of 8: sixteen bytes of gate and of up per thread.
+__global__ void gelu_gate_vec_kernel(const bf16_t* __restrict__ in, bf16_t* __restrict__ out, int inner8, size_t total8) {
+  for (size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x; idx < total8; idx += (size_t)gridDim.x * blockDim.x) {
+    const size_t t = idx / inner8, j = idx - t * inner8;
+    const uint4* row = reinterpret_cast<const uint4*>(in) + t * 2 * inner8;
+    float g[8], u[8], v[8];
+    rt_unpack8(row[j], g);
+    rt_unpack8(row[inner8 + j], u);
+#pragma unroll
+    for (int k = 0; k < 8; ++k) v[k] = rt_gelu_tanh(g[k]) * u[k];
+    reinterpret_cast<uint4*>(out)[idx] = rt_pack8(v);
+  }
+}
+
 static inline int rt_blocks(size_t total) { return (int)((total + 255) / 256 < 65535 ? (total + 255) / 256 : 65535); }
 
 extern "C" int ta_route_top(const void* logits, int n_tokens, int n_experts, int top, void* chosen, void* weights,
@@ -118,6 +181,12 @@ extern "C" int ta_expert_gate(const void* gate_up, const void* chosen, const voi
   const size_t total = (size_t)n_tokens * columns;
   if (total == 0) return 0;
   if (columns < n_experts * inner + shared) return -1;
+  if (dtype == DT_BF16 && inner % 8 == 0 && shared % 8 == 0 && columns % 8 == 0 &&
+      (((uintptr_t)gate_up | (uintptr_t)out) & 15) == 0) {
+    expert_gate_vec_kernel<<<rt_blocks(total / 8), 256, 0, stream>>>((const bf16_t*)gate_up, (const int*)chosen,
+        (const float*)weights, top, n_experts, inner, shared, columns, (bf16_t*)out, total / 8);
+    return LAUNCH_STATUS();
+  }
   if (dtype == DT_F32)
     expert_gate_kernel<float><<<rt_blocks(total), 256, 0, stream>>>((const float*)gate_up, (const int*)chosen,
         (const float*)weights, top, n_experts, inner, shared, columns, (float*)out, total);
@@ -144,6 +213,10 @@ extern "C" int ta_side_gate(const void* gate, const void* table, int table_width
 extern "C" int ta_gelu_gate(const void* in, void* out, int n_tokens, int inner, int dtype, hipStream_t stream) {
   const size_t total = (size_t)n_tokens * inner;
   if (total == 0) return 0;
+  if (dtype == DT_BF16 && inner % 8 == 0 && (((uintptr_t)in | (uintptr_t)out) & 15) == 0) {
+    gelu_gate_vec_kernel<<<rt_blocks(total / 8), 256, 0, stream>>>((const bf16_t*)in, (bf16_t*)out, inner / 8, total / 8);
+    return LAUNCH_STATUS();
+  }
   if (dtype == DT_F32)
     gelu_gate_kernel<float><<<rt_blocks(total), 256, 0, stream>>>((const float*)in, (float*)out, inner, total);
   else
