@@ -421,7 +421,8 @@ CUTS = {"prompt": lambda n: [n], "portions": lambda n: [37, 2, 16, 1, 1, 29] + [
 @pytest.mark.parametrize("cut", list(CUTS))
 @pytest.mark.parametrize("n_q,n_k,share,d,dv,size,keep", [(4, 2, 1, 16, 24, 40, 20), (4, 4, 2, 16, 8, 23, 0), (6, 2, 1, 32, 32, 16, 17),
                                                          (8, 2, 2, 64, 64, 33, 0), (2, 1, 1, 48, 48, 64, 5), (3, 3, 1, 12, 14, 1, 3),
-                                                         (4, 2, 1, 64, 64, 24, 70), (4, 1, 1, 128, 128, 9, 100), (4, 4, 2, 32, 32, 20, 0)])
+                                                         (4, 2, 1, 64, 64, 24, 70), (4, 1, 1, 128, 128, 9, 100), (4, 4, 2, 32, 32, 20, 0),
+                                                         (2, 2, 1, 32, 32, 5, 140)])
 def test_one_key_made_to_stand_out_at_every_edge(backend, cut, n_q, n_k, share, d, dv, size, keep):
     """Every query is made to score one chosen key far above all others: the key just inside its window, just outside
     it, the last kept first position, the one behind it, the keys on either side of a page border, a key far back and
