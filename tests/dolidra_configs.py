@@ -85,10 +85,11 @@ DOLIDRA = {
 }
 
 
-def write_model(raw: dict, seed: int, folder: str, sharpen: float = 6.0) -> str:
+def write_model(raw: dict, seed: int, folder: str, sharpen: float = 6.0, router: float = 0.4) -> str:
     """A model folder from the random-weights mode, with its matrices made `sharpen` times larger, so that attention
     weights are peaked: a key too many or too few, a window one position off or a lost kept key then moves the logits
-    by much more than rounding does.  The routers stay soft (several experts carry weight), the vectors behind the
+    by much more than rounding does.  The routers stay soft (`router` times the drawn weights: several experts carry
+    weight; a large factor makes the choice decisive instead, far from the near ties that rounding tips), the vectors behind the
     differential factor are made large enough for it to differ from layer to layer, and the embedding is of the size
     of what the layers add."""
     import tokenizer_amd as ta
@@ -104,8 +105,54 @@ def write_model(raw: dict, seed: int, folder: str, sharpen: float = 6.0) -> str:
         elif name.endswith((".lq1", ".lk1", ".lq2", ".lk2")):
             tensors[name] = (tensor.float() * 4.0).to(torch.bfloat16)
         elif name.endswith(".router"):
-            tensors[name] = (tensor.float() * 0.4).to(torch.bfloat16)
+            tensors[name] = (tensor.float() * router).to(torch.bfloat16)
         elif tensor.dim() == 2 and name not in ("head", "side.embed"):
             tensors[name] = (tensor.float() * sharpen).to(torch.bfloat16)
     save_file(tensors, path)
     return folder
+
+
+def random_config(seed: int) -> dict:
+    """A Dolidra configuration drawn from a seed: the number and order of layers, both kinds of attention, head counts and
+    groupings, key and value sizes (some in sixteens, some odd multiples of two), windows, kept positions, rotated
+    coordinates with and without scaling, dense and routed feed-forwards, layers without one, a loop or none, a token
+    input or none."""
+    import random
+    rng = random.Random(seed)
+    width = rng.choice([32, 40, 64, 72, 96, 128])
+    layers = []
+    for _ in range(rng.randint(1, 4)):
+        kv_heads = rng.choice([1, 1, 2, 3])
+        heads = kv_heads * rng.choice([1, 2, 4])
+        dim = rng.choice([8, 12, 16, 16, 32, 32, 48, 64])
+        vdim = dim if rng.random() < 0.6 else rng.choice([8, 10, 16, 24, 40])
+        size = rng.choice([None, 1, 2, 7, 16, 17, 31, 40, 64, 100])
+        rot = None
+        if rng.random() < 0.85:
+            dims = rng.choice([dim, dim, dim // 2, max(2, dim // 4 // 2 * 2), 2])
+            scaling = None
+            if rng.random() < 0.5:
+                scaling = (rng.choice([2.0, 4.0, 8.0]), 1.0, rng.choice([2.0, 4.0]), rng.choice([16, 64, 256, 2048]))
+            rot = _rot(dims, rng.choice([100.0, 10000.0, 250000.0]), scaling)
+        scale = rng.choice([dim ** -0.5, 0.2, 0.35])
+        if rng.random() < 0.5:
+            mixer = _differential(heads, kv_heads, dim, vdim, size, scale, rng.choice([0.0, 0.2, 0.5, 0.8]), rot)
+        else:
+            mixer = _gated(heads, kv_heads, dim, vdim, size, rng.choice([0, 1, 5, 16, 20, 33, 70]), scale, rot)
+        kind = rng.random()
+        if kind < 0.15:
+            mlp = None
+        elif kind < 0.55:
+            mlp = _dense(rng.choice([24, 50, 64, 100]))
+        else:
+            experts = rng.choice([1, 2, 4, 6, 9])
+            mlp = _moe(experts, rng.randint(1, min(experts, 3)), rng.choice([8, 10, 24, 32]), rng.choice([None, None, 6, 16]))
+        layers.append(_layer(mixer, mlp))
+    raw = {"architecture": "Dolidra", "vocab": rng.choice([97, 128, 211, 300]), "width": width,
+           "norm": {"eps": rng.choice([1e-5, 1e-6, 3e-6])}, "layers": layers}
+    if rng.random() < 0.7:
+        start = rng.randint(0, len(layers) - 1)
+        raw["loop"] = {"start": start, "stop": rng.randint(start, len(layers)), "times": rng.randint(1, 3)}
+    if rng.random() < 0.7:
+        raw["token_side"] = {"dim": rng.choice([1, 3, 4, 8, 16, 24])}
+    return raw
