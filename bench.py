@@ -272,28 +272,30 @@ def dolidra_config(sizes: dict, layers: int, window: int = 4096, keep_first: int
     maps each, so that queries and keys are as wide as Qwen2's; the windows are longer than the bench's contexts, so
     that both models' attention reads the same keys; a routed feed-forward has `experts` experts of a quarter of the
     dense inner width, of which a token uses `top`, and a shared expert of half of it (as many multiply-adds a token
-    as the dense one).  The layers alternate as differential + dense, differential + routed, gated + dense,
-    differential + routed, and the first two run twice."""
+    as the dense one).  The layers alternate as differential + dense, gated + routed, differential + routed,
+    gated + dense, and the second and third run twice."""
     width, heads, kv_heads = sizes["hidden_size"], sizes["num_attention_heads"], sizes["num_key_value_heads"]
     d, inner = width // heads, sizes["intermediate_size"]
     rot = {"base": float(sizes.get("rope_theta", 1e6)), "dims": d,
-           "scaling": {"factor": 4.0, "low": 1.0, "high": 4.0, "original": 8192}}
+           "scaling": {"factor": 8.0, "low": 1.0, "high": 4.0, "original": 8192}}
     dense = {"kind": "dense", "ff": inner}
     routed = {"kind": "moe", "expert": {"ff": inner // 4 // 8 * 8}, "router": {"experts": experts, "top": top},
               "shared": {"ff": inner // 2 // 8 * 8}}
     out = []
     for index in range(layers):
         kind = index % 4
-        if kind == 2:
+        mlp = routed if kind in (1, 2) else dense
+        if kind in (1, 3):
             mixer = {"heads": heads, "kv_heads": kv_heads, "dim": d, "vdim": d, "scale": d ** -0.5,
                      "mask": {"size": window, "keep_first": keep_first}, "rot": {"base": rot["base"], "dims": d // 4}}
-            out.append({"type": "attention_2", "mixer": mixer, "mlp": dense})
+            out.append({"type": "attention_2", "mixer": mixer, "mlp": mlp})
             continue
         mixer = {"heads": max(1, heads // 2), "kv_heads": max(1, kv_heads // 2), "dim": d, "vdim": d, "scale": d ** -0.5,
-                 "diff": 0.5, "mask": {"size": window}, "rot": rot}
-        out.append({"type": "attention", "mixer": mixer, "mlp": dense if kind == 0 else routed})
+                 "diff": 0.4, "mask": {"size": window}, "rot": rot}
+        out.append({"type": "attention", "mixer": mixer, "mlp": mlp})
+    loop = {"start": 1, "stop": 3, "times": 2} if layers >= 3 else {"start": 0, "stop": layers, "times": 2}
     return {"architecture": "Dolidra", "vocab": sizes["vocab_size"], "width": width, "norm": {"eps": 1e-6},
-            "token_side": {"dim": 16}, "loop": {"start": 0, "stop": min(2, layers), "times": 2}, "layers": out}
+            "token_side": {"dim": 16}, "loop": loop, "layers": out}
 
 
 def run_design(args, sizes: dict) -> dict:

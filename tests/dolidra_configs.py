@@ -72,15 +72,15 @@ DOLIDRA = {
     # and kept positions that cut tiles of sixteen tokens and pages of sixteen.
     "D": ({"architecture": "Dolidra", "vocab": 180, "width": 128, "norm": {"eps": 1e-6}, "token_side": {"dim": 8},
            "loop": {"start": 0, "stop": 2, "times": 2},
-           "layers": [_layer(_differential(4, 2, 32, 32, 40, 0.2, 0.5, _rot(32, 250000.0)), _dense(96)),
-                      _layer(_gated(4, 2, 64, 64, 48, 16, 0.125, _rot(16, 250000.0)), _moe(8, 2, 32, shared=64)),
+           "layers": [_layer(_differential(4, 2, 32, 32, 36, 0.2, 0.45, _rot(32, 500000.0)), _dense(96)),
+                      _layer(_gated(4, 2, 64, 64, 48, 16, 0.125, _rot(16, 500000.0)), _moe(8, 2, 32, shared=64)),
                       _layer(_gated(2, 1, 16, 16, 19, 7, 0.25, _rot(16, 1000.0)), _dense(80)),
                       _layer(_differential(8, 1, 16, 16, 23, 0.25, 0.35, _rot(8, 1000.0)), _moe(4, 2, 48))]}, 34),
     # Windows of hundreds of positions with kept first positions far behind them.
     "E": ({"architecture": "Dolidra", "vocab": 260, "width": 128, "norm": {"eps": 1e-6}, "token_side": {"dim": 16},
            "loop": {"start": 1, "stop": 2, "times": 2},
-           "layers": [_layer(_differential(4, 2, 32, 32, 300, 0.18, 0.5, _rot(32, 250000.0, (4.0, 1.0, 4.0, 2048))), _dense(96)),
-                      _layer(_gated(4, 2, 32, 32, 260, 40, 0.18, _rot(8, 250000.0)), _moe(6, 2, 32, shared=32)),
+           "layers": [_layer(_differential(4, 2, 32, 32, 300, 0.18, 0.6, _rot(32, 80000.0, (8.0, 1.0, 4.0, 1024))), _dense(96)),
+                      _layer(_gated(4, 2, 32, 32, 260, 44, 0.18, _rot(8, 80000.0)), _moe(6, 2, 32, shared=32)),
                       _layer(_gated(2, 2, 64, 64, 520, 3, 0.125, _rot(64, 10000.0)), _dense(64))]}, 55),
 }
 
@@ -126,14 +126,14 @@ def random_config(seed: int) -> dict:
         heads = kv_heads * rng.choice([1, 2, 4])
         dim = rng.choice([8, 12, 16, 16, 32, 32, 48, 64])
         vdim = dim if rng.random() < 0.6 else rng.choice([8, 10, 16, 24, 40])
-        size = rng.choice([None, 1, 2, 7, 16, 17, 31, 40, 64, 100])
+        size = rng.choice([None, 1, 2, 7, 16, 17, 31, 36, 64, 100])
         rot = None
         if rng.random() < 0.85:
             dims = rng.choice([dim, dim, dim // 2, max(2, dim // 4 // 2 * 2), 2])
             scaling = None
             if rng.random() < 0.5:
-                scaling = (rng.choice([2.0, 4.0, 8.0]), 1.0, rng.choice([2.0, 4.0]), rng.choice([16, 64, 256, 2048]))
-            rot = _rot(dims, rng.choice([100.0, 10000.0, 250000.0]), scaling)
+                scaling = (rng.choice([2.0, 4.0, 8.0]), 1.0, rng.choice([2.0, 4.0]), rng.choice([16, 64, 256, 1024]))
+            rot = _rot(dims, rng.choice([100.0, 10000.0, 500000.0]), scaling)
         scale = rng.choice([dim ** -0.5, 0.2, 0.35])
         if rng.random() < 0.5:
             mixer = _differential(heads, kv_heads, dim, vdim, size, scale, rng.choice([0.0, 0.2, 0.5, 0.8]), rot)
