@@ -305,7 +305,7 @@ class Batch:
 
 
 @pytest.mark.parametrize("backend", BACKENDS)
-@pytest.mark.parametrize("width", [64, 52, 200, 4352])
+@pytest.mark.parametrize("width", [64, 52, 50, 200, 2050, 4352])
 def test_the_norm_behind_a_sub_layer_with_the_add_and_the_next_norm(backend, width):
     ops, device, dtype = ops_for(backend)
     gen = torch.Generator().manual_seed(width)
