@@ -510,6 +510,10 @@ def test_routing_and_the_experts(backend, experts, top, inner, shared, width):
     picked, order = torch.topk(exact, top, dim=-1)
     assert torch.equal(chosen.cpu().long(), order)
     assert float((weights.double().cpu() - torch.softmax(picked, dim=-1)).abs().max()) <= 1e-5
+    if hasattr(ops, "route_rows") and width % 8 == 0:      # the product and the choice in one kernel
+        again, weights_again = torch.full_like(chosen, -1), torch.zeros_like(weights)
+        assert ops.route_rows(dev(h), dev(w["router"]), again, weights_again)
+        assert torch.equal(again, chosen) and float((weights_again - weights).abs().max()) <= 1e-5
     gate_up = ops.linear(dev(h), dev(torch.cat([w[f"{name}.{part}"] for name in names for part in ("gate", "up")])))
     fill = (-(experts * inner + shared)) % 8
     act = torch.full((tokens, experts * inner + shared + fill), float("nan"), dtype=dtype, device=device)

@@ -45,6 +45,101 @@ route_top_kernel(const float* __restrict__ logits, int n_tokens, int n_experts, 
   if (lane < top) weights[(size_t)t * top + lane] = mine / total;
 }
 
+// Eight bfloat16 elements (sixteen bytes) as floats, and back.
+__device__ __forceinline__ void rt_unpack8(const uint4 raw, float (&v)[8]) {
+  const uint32_t w[4] = {raw.x, raw.y, raw.z, raw.w};
+#pragma unroll
+  for (int i = 0; i < 4; ++i) { v[2 * i] = __uint_as_float(w[i] << 16); v[2 * i + 1] = __uint_as_float(w[i] & 0xffff0000u); }
+}
+__device__ __forceinline__ uint4 rt_pack8(const float (&v)[8]) {
+  uint32_t w[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) w[i] = (uint32_t)float_to_bf16_bits(v[2 * i]) | ((uint32_t)float_to_bf16_bits(v[2 * i + 1]) << 16);
+  return make_uint4(w[0], w[1], w[2], w[3]);
+}
+
+#define RT_MAX_EXPERTS 256
+#define RT_ROW_PIECES 8        // sixteen-byte pieces of a row that a lane keeps: rows of up to 64 * 8 * 8 bfloat16 elements
+
+template <typename T> struct RtVec;
+template <> struct RtVec<bf16_t> {
+  static constexpr int N = 8;
+  __device__ static __forceinline__ void load(const bf16_t* p, float (&v)[8]) { rt_unpack8(*reinterpret_cast<const uint4*>(p), v); }
+};
+template <> struct RtVec<float> {
+  static constexpr int N = 4;
+  __device__ static __forceinline__ void load(const float* p, float (&v)[4]) {
+    const float4 raw = *reinterpret_cast<const float4*>(p);
+    v[0] = raw.x; v[1] = raw.y; v[2] = raw.z; v[3] = raw.w;
+  }
+};
+
+// The router's product and the choice in one kernel, a workgroup a token: x [n_tokens, hidden] (row stride lda) and
+// router [n_experts, hidden] of type T in pieces of sixteen bytes; wave w forms the logits of experts w, w + 4, ... as
+// float sums (a lane keeps its pieces of the row), wave 0 then picks as route_top_kernel does.
+template <typename T>
+__global__ void __launch_bounds__(256)
+route_rows_kernel(const T* __restrict__ x, int lda, const T* __restrict__ router, int hidden, int n_experts, int top,
+                  int* __restrict__ chosen, float* __restrict__ weights) {
+  constexpr int N = RtVec<T>::N;
+  __shared__ float logit_s[RT_MAX_EXPERTS];
+  const int t = blockIdx.x;
+  const int lane = threadIdx.x & (WAVE - 1), wave = threadIdx.x / WAVE;
+  const T* row = x + (size_t)t * lda;
+  float xv[RT_ROW_PIECES][N];
+#pragma unroll
+  for (int p = 0; p < RT_ROW_PIECES; ++p) {
+    const int at = (p * WAVE + lane) * N;
+    if (at < hidden) RtVec<T>::load(row + at, xv[p]);
+    else
+#pragma unroll
+      for (int k = 0; k < N; ++k) xv[p][k] = 0.f;
+  }
+  for (int e = wave; e < n_experts; e += 256 / WAVE) {
+    const T* w = router + (size_t)e * hidden;
+    float sum = 0.f;
+#pragma unroll
+    for (int p = 0; p < RT_ROW_PIECES; ++p) {
+      const int at = (p * WAVE + lane) * N;
+      if (at < hidden) {
+        float wv[N];
+        RtVec<T>::load(w + at, wv);
+#pragma unroll
+        for (int k = 0; k < N; ++k) sum = fmaf(wv[k], xv[p][k], sum);
+      }
+    }
+    sum = wave_sum(sum);
+    if (lane == 0) logit_s[e] = sum;
+  }
+  __syncthreads();
+  if (wave != 0) return;
+  float top_value = 0.f, total = 0.f, mine = 0.f, last_value = INFINITY;
+  int last = -1;
+  for (int k = 0; k < top; ++k) {
+    float best = -INFINITY;
+    int best_at = n_experts;
+    for (int e = lane; e < n_experts; e += WAVE) {
+      const float v = logit_s[e];
+      const bool behind = v < last_value || (v == last_value && e > last);
+      if (behind && (v > best || (v == best && e < best_at))) { best = v; best_at = e; }
+    }
+#pragma unroll
+    for (int off = WAVE / 2; off > 0; off >>= 1) {
+      const float other = __shfl_xor(best, off, WAVE);
+      const int other_at = __shfl_xor(best_at, off, WAVE);
+      if (other > best || (other == best && other_at < best_at)) { best = other; best_at = other_at; }
+    }
+    if (k == 0) top_value = best;
+    const float term = expf(best - top_value);
+    total += term;
+    if (lane == k) mine = term;
+    if (lane == 0) chosen[(size_t)t * top + k] = best_at;
+    last = best_at;
+    last_value = best;
+  }
+  if (lane < top) weights[(size_t)t * top + lane] = mine / total;
+}
+
 // gate_up: [n_tokens, n_experts * 2 * inner + 2 * shared], expert e's gate rows then its up rows, the shared expert
 // last.  out: [n_tokens, columns] with columns >= n_experts * inner + shared: out[t, e * inner + i] =
 // w * silu(gate) * up for an expert the token chose with weight w, 0 for the others; the shared expert's columns
@@ -100,19 +195,6 @@ __global__ void gelu_gate_kernel(const T* __restrict__ in, T* __restrict__ out, 
     const int j = (int)(idx - t * inner);
     st(out + idx, rt_gelu_tanh(ld(in + t * 2 * inner + j)) * ld(in + t * 2 * inner + inner + j));
   }
-}
-
-// Eight bfloat16 elements (sixteen bytes) as floats, and back.
-__device__ __forceinline__ void rt_unpack8(const uint4 raw, float (&v)[8]) {
-  const uint32_t w[4] = {raw.x, raw.y, raw.z, raw.w};
-#pragma unroll
-  for (int i = 0; i < 4; ++i) { v[2 * i] = __uint_as_float(w[i] << 16); v[2 * i + 1] = __uint_as_float(w[i] & 0xffff0000u); }
-}
-__device__ __forceinline__ uint4 rt_pack8(const float (&v)[8]) {
-  uint32_t w[4];
-#pragma unroll
-  for (int i = 0; i < 4; ++i) w[i] = (uint32_t)float_to_bf16_bits(v[2 * i]) | ((uint32_t)float_to_bf16_bits(v[2 * i + 1]) << 16);
-  return make_uint4(w[0], w[1], w[2], w[3]);
 }
 
 // expert_gate for bfloat16 with inner, shared and columns multiples of 8: a thread makes eight columns, which lie in
@@ -173,6 +255,24 @@ extern "C" int ta_route_top(const void* logits, int n_tokens, int n_experts, int
   if (top <= 0 || top > n_experts || top > WAVE) return -1;
   route_top_kernel<<<(n_tokens + 3) / 4, 256, 0, stream>>>((const float*)logits, n_tokens, n_experts, top, (int*)chosen,
                                                            (float*)weights);
+  return LAUNCH_STATUS();
+}
+
+// Returns -2 for sizes the fused kernel does not take (the caller then forms the logits with a product of its own).
+extern "C" int ta_route_rows(const void* x, int lda, const void* router, int n_tokens, int hidden, int n_experts, int top,
+                             void* chosen, void* weights, int dtype, hipStream_t stream) {
+  if (n_tokens <= 0) return 0;
+  if (top <= 0 || top > n_experts || top > WAVE) return -1;
+  const int piece = dtype == DT_F32 ? 4 : 8;
+  if (n_experts > RT_MAX_EXPERTS || hidden % piece || lda % piece || hidden > WAVE * RT_ROW_PIECES * piece ||
+      (((uintptr_t)x | (uintptr_t)router) & 15))
+    return -2;
+  if (dtype == DT_F32)
+    route_rows_kernel<float><<<n_tokens, 256, 0, stream>>>((const float*)x, lda, (const float*)router, hidden, n_experts, top,
+                                                           (int*)chosen, (float*)weights);
+  else
+    route_rows_kernel<bf16_t><<<n_tokens, 256, 0, stream>>>((const bf16_t*)x, lda, (const bf16_t*)router, hidden, n_experts,
+                                                            top, (int*)chosen, (float*)weights);
   return LAUNCH_STATUS();
 }
 

@@ -155,7 +155,7 @@ class Ops:
                      "ta_sample_workspace_words", "ta_library_gemm_bf16", "ta_compute_units", "ta_read_stream",
                      "ta_embedding_streams", "ta_streams_step", "ta_token_shift", "ta_mlstm_scan", "ta_mlstm_chunked", "ta_head_norm_gate",
                      "ta_capped_gate", "ta_norm_add_rmsnorm", "ta_norm_rotate_store", "ta_differential_heads",
-                     "ta_sigmoid_head_gate", "ta_route_top", "ta_expert_gate", "ta_side_gate", "ta_gelu_gate", "ta_norm_side_norm"):
+                     "ta_sigmoid_head_gate", "ta_route_top", "ta_expert_gate", "ta_side_gate", "ta_gelu_gate", "ta_norm_side_norm", "ta_route_rows"):
             getattr(self.lib, name).restype = ctypes.c_int
         self.lib.ta_library_gemm_bf16.argtypes = [ctypes.c_void_p] * 4 + [ctypes.c_int] * 5 + [
             ctypes.c_void_p, ctypes.c_size_t, ctypes.c_int, ctypes.c_void_p]
@@ -399,6 +399,25 @@ class Ops:
         _need(0 < top <= min(n_experts, 64), "between one and 64 experts a token, no more than there are")
         self._check(self.lib.ta_route_top(_ptr(logits), n_tokens, n_experts, top, _ptr(chosen), _ptr(weights), self._stream()),
                     "route_top")
+
+    def route_rows(self, x: torch.Tensor, router: torch.Tensor, chosen: torch.Tensor, weights: torch.Tensor) -> bool:
+        """`route_top` of the float32 logits x @ router.T without leaving them in memory: product and choice in one
+        kernel.  x [T, H], router [E, H] of one dtype.  Returns False for sizes the kernel does not take (more than 256
+        experts, rows that are not whole pieces of sixteen bytes or longer than 4,096 bfloat16 / 2,048 float32
+        elements): the caller then forms the logits with `linear` and calls `route_top`."""
+        _dev(x, router, chosen, weights)
+        n_tokens, hidden = x.shape
+        n_experts, top = router.shape[0], chosen.shape[1]
+        _need(x.dtype == router.dtype and x.stride(1) == 1 and router.is_contiguous() and router.shape[1] == hidden, "router [E, H]")
+        _need(chosen.dtype == torch.int32 and weights.dtype == torch.float32 and chosen.is_contiguous() and weights.is_contiguous()
+              and tuple(chosen.shape) == (n_tokens, top) == tuple(weights.shape), "chosen int32 and weights float32 [T, top]")
+        _need(0 < top <= min(n_experts, 64), "between one and 64 experts a token, no more than there are")
+        status = self.lib.ta_route_rows(_ptr(x), x.stride(0) if n_tokens > 1 else hidden, _ptr(router), n_tokens, hidden,
+                                        n_experts, top, _ptr(chosen), _ptr(weights), _code(x.dtype), self._stream())
+        if status == -2:
+            return False
+        self._check(status, "route_rows")
+        return True
 
     def expert_gate(self, gate_up: torch.Tensor, chosen: torch.Tensor, weights: torch.Tensor, n_experts: int, inner: int,
                     shared: int, out: torch.Tensor) -> torch.Tensor:

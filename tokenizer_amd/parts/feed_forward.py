@@ -136,10 +136,11 @@ class RoutedExperts(FeedForward):
 
     def forward(self, x, ctx):
         ops = self.runtime.ops
-        logits = ops.linear(x, self.w_router, out_dtype=torch.float32)
         chosen = torch.empty((x.shape[0], self.top_k), dtype=torch.int32, device=x.device)
         weights = torch.empty((x.shape[0], self.top_k), dtype=torch.float32, device=x.device)
-        ops.route_top(logits, chosen, weights)
+        fused = getattr(ops, "route_rows", None)          # the router's product and the choice in one kernel, where there is one
+        if fused is None or not fused(x, self.w_router, chosen, weights):
+            ops.route_top(ops.linear(x, self.w_router, out_dtype=torch.float32), chosen, weights)
         gate_up = ops.linear(x, self.w_gate_up)
         act = torch.empty((x.shape[0], self.columns), dtype=x.dtype, device=x.device)
         ops.expert_gate(gate_up, chosen, weights, self.n_experts, self.inner, self.shared, act)
