@@ -632,3 +632,18 @@ def first_near_tie(cfg, tensors, ids, within=0.08) -> int:
     finally:
         plain.routed_ff = routed
     return first[0]
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["A", "D"])
+def test_the_step_by_step_paths_behind_the_fused_kernels(folders, oracle, name, dtype, monkeypatch):
+    """Sizes the fused kernels do not take (rows of more than 4,096 elements, wide token inputs, hundreds of experts)
+    run the token input and the router step by step; here the fused kernels are made to decline."""
+    from tokenizer_amd.kernels import get_ops
+    ops = get_ops()
+    monkeypatch.setattr(ops, "norm_side_norm", lambda *args, **kw: None, raising=False)
+    monkeypatch.setattr(ops, "route_rows", lambda *args, **kw: False, raising=False)
+    reqs = requests_for(name, (33, 97, 21, 64, 50))
+    steps = tt.mixed(reqs, 5, max_live=3, tail=14)
+    check_trace(folders, oracle, name, "gpu-" + dtype, steps, reqs)
