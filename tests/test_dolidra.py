@@ -647,3 +647,49 @@ def test_the_step_by_step_paths_behind_the_fused_kernels(folders, oracle, name, 
     reqs = requests_for(name, (33, 97, 21, 64, 50))
     steps = tt.mixed(reqs, 5, max_live=3, tail=14)
     check_trace(folders, oracle, name, "gpu-" + dtype, steps, reqs)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("experts,top,inner,shared,width,tokens", [(8, 2, 32, 16, 64, 300), (4, 2, 24, 0, 72, 1200), (5, 3, 8, 8, 40, 77),
+                                                                  (12, 1, 16, 0, 64, 2100)])
+def test_routed_layers_over_sorted_tokens(experts, top, inner, shared, width, tokens, monkeypatch):
+    """The form that sorts a step's (token, expert) pairs into tiles of one expert each, against the plain function and
+    against the form that multiplies every token with every expert."""
+    from tokenizer_amd.kernels import get_ops
+    from tokenizer_amd.parts import FEED_FORWARDS, FeedForwardSpec, Runtime
+    device, dtype = torch.device("cuda:0"), torch.bfloat16
+    gen = torch.Generator().manual_seed(experts * tokens)
+    rand = lambda *shape: torch.randn(*shape, generator=gen, dtype=torch.float64)
+    h = rounded(rand(tokens, width), dtype)
+    w = {"router": rounded(rand(experts, width) * 0.5, dtype)}
+    for name in [f"e{j}" for j in range(experts)] + (["shared"] if shared else []):
+        size = shared if name == "shared" else inner
+        w.update({f"{name}.gate": rounded(rand(size, width) * 0.3, dtype), f"{name}.up": rounded(rand(size, width) * 0.3, dtype),
+                  f"{name}.down": rounded(rand(width, size) * 0.3, dtype)})
+    want = plain.routed_ff(h, w, {"router": {"experts": experts, "top": top}, "shared": {"ff": shared} if shared else None})
+    spec = FeedForwardSpec("routed_experts", hidden_size=width, intermediate_size=inner, n_experts=experts, top_k=top,
+                           shared_size=shared)
+    cls = FEED_FORWARDS.get("routed_experts")
+    part = cls(spec, {name: t.to(dtype).to(device).contiguous() for name, t in w.items()}, Runtime(dtype, device, get_ops()))
+    assert part.groupable
+    x = h.to(dtype).to(device)
+    monkeypatch.setattr(cls, "GROUPED_FROM", 1)
+    sorted_form = part.forward(x, None).double().cpu()
+    monkeypatch.setattr(cls, "GROUPED_FROM", 1 << 30)
+    every_expert = part.forward(x, None).double().cpu()
+    # (A token whose last chosen and best unchosen logit are nearly equal may go either way in either form: the two
+    # forms form the logits with the same kernel, so they agree with each other; the plain function may not.)
+    bound = 4e-2 * float(want.abs().max())
+    assert float((sorted_form - every_expert).abs().max()) <= bound
+    off = (sorted_form - want).abs().amax(dim=-1) > bound
+    assert int(off.sum()) <= max(1, tokens // 50)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("name", ["A", "D"])
+def test_sorted_routed_layers_through_the_engine(folders, oracle, name, monkeypatch):
+    from tokenizer_amd.parts import FEED_FORWARDS
+    monkeypatch.setattr(FEED_FORWARDS.get("routed_experts"), "GROUPED_FROM", 2)
+    reqs = requests_for(name, (33, 97, 21, 64, 50, 80))
+    steps = tt.mixed(reqs, 9, max_live=3, tail=14)
+    check_trace(folders, oracle, name, "gpu-bfloat16", steps, reqs)

@@ -155,8 +155,11 @@ class Ops:
                      "ta_sample_workspace_words", "ta_library_gemm_bf16", "ta_compute_units", "ta_read_stream",
                      "ta_embedding_streams", "ta_streams_step", "ta_token_shift", "ta_mlstm_scan", "ta_mlstm_chunked", "ta_head_norm_gate",
                      "ta_capped_gate", "ta_norm_add_rmsnorm", "ta_norm_rotate_store", "ta_differential_heads",
-                     "ta_sigmoid_head_gate", "ta_route_top", "ta_expert_gate", "ta_side_gate", "ta_gelu_gate", "ta_norm_side_norm", "ta_route_rows"):
+                     "ta_sigmoid_head_gate", "ta_route_top", "ta_expert_gate", "ta_side_gate", "ta_gelu_gate", "ta_norm_side_norm", "ta_route_rows", "ta_expert_slots", "ta_grouped_gemm_bf16", "ta_expert_combine"):
             getattr(self.lib, name).restype = ctypes.c_int
+        self.lib.ta_grouped_gemm_bf16.argtypes = [ctypes.c_void_p, ctypes.c_int, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int,
+                                                  ctypes.c_int, ctypes.c_void_p, ctypes.c_long, ctypes.c_int, ctypes.c_void_p,
+                                                  ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_void_p]
         self.lib.ta_library_gemm_bf16.argtypes = [ctypes.c_void_p] * 4 + [ctypes.c_int] * 5 + [
             ctypes.c_void_p, ctypes.c_size_t, ctypes.c_int, ctypes.c_void_p]
         self._workspaces: dict[int, torch.Tensor] = {}
@@ -418,6 +421,64 @@ class Ops:
             return False
         self._check(status, "route_rows")
         return True
+
+    # Routed feed-forwards over sorted tokens (bfloat16): tiles of `bm` slots that belong to one expert each.
+    GROUPED_EXPERTS = 256
+
+    @staticmethod
+    def grouped_tiles(n_entries: int, n_experts: int, bm: int) -> int:
+        """How many tiles of `bm` slots the (token, expert) pairs of a step can need at most."""
+        return -(-n_entries // bm) + n_experts
+
+    def expert_slots(self, chosen: torch.Tensor, n_experts: int, bm: int):
+        """Sort a step's picks (chosen int32 [T, top]) by expert into tiles of `bm` slots: returns (slot_of int32
+        [T * top], row_of int32 [tiles * bm] with -1 for slots that only fill a tile up, tile_expert int32 [tiles] with
+        -1 for tiles past the last run), all on the device; nothing comes back to the host."""
+        _dev(chosen)
+        _need(chosen.dtype == torch.int32 and chosen.dim() == 2 and chosen.is_contiguous(), "chosen is int32 [T, top]")
+        _need(0 < n_experts <= self.GROUPED_EXPERTS and bm in (64, 128), "up to 256 experts, tiles of 64 or 128 slots")
+        n_entries = chosen.numel()
+        tiles = self.grouped_tiles(n_entries, n_experts, bm)
+        slot_of = torch.empty(n_entries, dtype=torch.int32, device=chosen.device)
+        row_of = torch.empty(tiles * bm, dtype=torch.int32, device=chosen.device)
+        tile_expert = torch.empty(tiles, dtype=torch.int32, device=chosen.device)
+        self._check(self.lib.ta_expert_slots(_ptr(chosen), n_entries, chosen.shape[1], n_experts, bm, tiles, _ptr(slot_of),
+                                             _ptr(row_of), _ptr(tile_expert), self._stream()), "expert_slots")
+        return slot_of, row_of, tile_expert
+
+    def grouped_linear(self, x: torch.Tensor, row_of: torch.Tensor | None, tile_expert: torch.Tensor, bm: int,
+                       weight: torch.Tensor, expert_stride: int, n_out: int, k: int, out_dtype: torch.dtype) -> torch.Tensor:
+        """out[slot] = x[row_of[slot]] (or x[slot] without `row_of`) @ W_e.T for every slot of every tile, W_e the
+        [n_out, k] block of `weight` (contiguous [rows, ldw]) that starts `expert_stride` elements times the tile's
+        expert into it.  bfloat16 operands, float32 sums; out [tiles * bm, n_out] bfloat16 or float32."""
+        _dev(x, row_of, tile_expert, weight)
+        tiles = tile_expert.numel()
+        _need(x.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16 and x.stride(1) == 1 and weight.is_contiguous(),
+              "bfloat16 operands with contiguous rows")
+        _need(x.shape[1] >= k and (row_of is not None or x.shape[0] >= tiles * bm), "rows of x for every slot")
+        _need(row_of is None or (row_of.dtype == torch.int32 and row_of.numel() == tiles * bm), "row_of is int32 [tiles bm]")
+        _need(tile_expert.dtype == torch.int32 and k % 8 == 0 and x.stride(0) % 8 == 0 and weight.shape[1] % 8 == 0
+              and expert_stride % 8 == 0, "K, strides and the experts' offsets in eights")
+        out = torch.empty((tiles * bm, n_out), dtype=out_dtype, device=x.device)
+        self._check(self.lib.ta_grouped_gemm_bf16(_ptr(x), x.stride(0), _ptr(row_of), _ptr(tile_expert), tiles, bm, _ptr(weight),
+                                                  int(expert_stride), weight.shape[1], _ptr(out), n_out, n_out, k,
+                                                  _code(out_dtype), self._stream()), "grouped_linear")
+        return out
+
+    def expert_combine(self, rows: torch.Tensor, slot_of: torch.Tensor, weights: torch.Tensor, shared: torch.Tensor | None,
+                       out: torch.Tensor) -> torch.Tensor:
+        """out[t] = shared[t] (if given) + sum over the token's picks of weights[t, k] * rows[slot_of[t top + k]]; rows
+        float32 [slots, H], weights float32 [T, top], shared and out [T, H] of one dtype."""
+        _dev(rows, slot_of, weights, shared, out)
+        n_tokens, top = weights.shape
+        _need(rows.dtype == torch.float32 and rows.is_contiguous() and rows.shape[1] == out.shape[1], "rows are float32 [slots, H]")
+        _need(slot_of.dtype == torch.int32 and slot_of.numel() == n_tokens * top and weights.dtype == torch.float32
+              and weights.is_contiguous(), "slot_of int32 [T top], weights float32 [T, top]")
+        _need(out.is_contiguous() and out.shape[0] == n_tokens and (shared is None or (shared.shape == out.shape
+              and shared.dtype == out.dtype and shared.is_contiguous())), "shared and out are [T, H]")
+        self._check(self.lib.ta_expert_combine(_ptr(rows), _ptr(slot_of), _ptr(weights), n_tokens, top, _ptr(shared), _ptr(out),
+                                               out.shape[1], _code(out.dtype), self._stream()), "expert_combine")
+        return out
 
     def expert_gate(self, gate_up: torch.Tensor, chosen: torch.Tensor, weights: torch.Tensor, n_experts: int, inner: int,
                     shared: int, out: torch.Tensor) -> torch.Tensor:

@@ -96,10 +96,15 @@ class RoutedExperts(FeedForward):
     All experts' gate and up matrices are one matrix, and all down matrices one matrix along K, so a step is two
     products whatever the routing: between them a kernel turns gate and up into weight * silu(gate) * up for the
     experts a token chose and into zero for the others (the shared expert counts as chosen with weight 1), and the
-    second product then adds the chosen experts' outputs up in its own sum.  The routing stays on the device, so
-    the step's launches do not depend on it.
+    second product then adds the chosen experts' outputs up in its own sum.  That multiplies every token with every
+    expert, which is right while the weights bound the step (few rows: every expert is read anyway).  Steps with
+    `GROUPED_FROM` or more (token, expert) pairs in bfloat16 sort the pairs by expert on the device into tiles of rows
+    that belong to one expert each, multiply every tile with its expert's matrices alone, and add a token's experts
+    up at the end (the shared expert runs as a dense one).  Either way the routing stays on the device, so the step's
+    launches do not depend on it.
     """
     graph_safe = True
+    GROUPED_FROM = 1024        # (token, expert) pairs from which the sorted form runs
 
     def __init__(self, spec: FeedForwardSpec, tensors: dict[str, torch.Tensor], runtime: Runtime):
         if spec.activation != "silu":
@@ -122,6 +127,13 @@ class RoutedExperts(FeedForward):
         self.w_gate_up = torch.cat(gate_up, dim=0).contiguous()
         self.w_down = torch.cat(down, dim=1).contiguous()
         self.columns = self.total + fill
+        # For the sorted form: the shared expert's matrices by themselves (views of the joined gate/up rows; its down
+        # columns as a matrix of their own).
+        self.groupable = (runtime.dtype == torch.bfloat16 and self.inner % 8 == 0 and spec.hidden_size % 8 == 0
+                          and self.shared % 8 == 0 and self.n_experts <= 256)
+        if self.groupable and self.shared:
+            self.w_shared_gate_up = self.w_gate_up[self.n_experts * 2 * self.inner:]
+            self.w_shared_down = self.w_down[:, self.n_experts * self.inner:self.n_experts * self.inner + self.shared].contiguous()
 
     @staticmethod
     def tensor_specs(spec: FeedForwardSpec) -> dict[str, TensorSpec]:
@@ -141,7 +153,26 @@ class RoutedExperts(FeedForward):
         fused = getattr(ops, "route_rows", None)          # the router's product and the choice in one kernel, where there is one
         if fused is None or not fused(x, self.w_router, chosen, weights):
             ops.route_top(ops.linear(x, self.w_router, out_dtype=torch.float32), chosen, weights)
+        if self.groupable and x.shape[0] * self.top_k >= self.GROUPED_FROM and hasattr(ops, "grouped_linear"):
+            return self._sorted(x, chosen, weights)
         gate_up = ops.linear(x, self.w_gate_up)
         act = torch.empty((x.shape[0], self.columns), dtype=x.dtype, device=x.device)
         ops.expert_gate(gate_up, chosen, weights, self.n_experts, self.inner, self.shared, act)
         return ops.linear(act, self.w_down)
+
+    def _sorted(self, x, chosen, weights):
+        """Tiles of rows that belong to one expert each: gate/up, the activation, down, then a token's experts added up."""
+        ops = self.runtime.ops
+        hidden, inner = x.shape[1], self.inner
+        bm = 128 if x.shape[0] * self.top_k >= 2048 * max(1, self.n_experts // 8) else 64
+        slot_of, row_of, tile_expert = ops.expert_slots(chosen, self.n_experts, bm)
+        gate_up = ops.grouped_linear(x, row_of, tile_expert, bm, self.w_gate_up, 2 * inner * hidden, 2 * inner, hidden,
+                                     torch.bfloat16)
+        act = torch.empty((gate_up.shape[0], inner), dtype=x.dtype, device=x.device)
+        ops.silu_gate(gate_up, act)
+        rows = ops.grouped_linear(act, None, tile_expert, bm, self.w_down, inner, hidden, inner, torch.float32)
+        shared = None
+        if self.shared:
+            shared = ops.linear(ops.linear_silu_gate(x, self.w_shared_gate_up), self.w_shared_down)
+        out = torch.empty((x.shape[0], hidden), dtype=x.dtype, device=x.device)
+        return ops.expert_combine(rows, slot_of, weights, shared, out)
